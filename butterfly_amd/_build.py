@@ -28,6 +28,7 @@ PKG = ROOT / "butterfly_amd"
 CSRC = ROOT / "csrc"
 OBJ = ROOT / "build" / "obj"
 ARCH = os.environ.get("BFLY_OFFLOAD_ARCH", "gfx950")
+PRECISE_KERNELS = {"gemm_any", "hyper", "mixers"}
 HIPCC = os.environ.get("HIPCC", shutil.which("hipcc") or "/opt/rocm/bin/hipcc")
 
 
@@ -80,14 +81,20 @@ def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = True) -> P
               "-D__HIP_PLATFORM_AMD__=1"]
     # fast-math for contraction / reassociation, but infinities stay meaningful: the attention
     # kernels use -inf as the empty-score sentinel
-    kflags = [HIPCC, f"--offload-arch={ARCH}", "-ffast-math", "-fno-finite-math-only", "-fno-gpu-rdc", *common]
+    # packed-FP32 VALU forms stay off: the compiler then emits scalar f32 arithmetic only
+    kflags = [HIPCC, f"--offload-arch={ARCH}", "-ffast-math", "-fno-finite-math-only", "-fno-gpu-rdc",
+              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", *common]
     # Host-only C++ for the bindings: ROCm's clang (x86 __bf16 support, libstdc++ ABI).
     hostcxx = os.environ.get("BFLY_HOST_CXX", "/opt/rocm/lib/llvm/bin/clang++")
     bflags = [hostcxx, "-x", "c++", *common, "-I/opt/rocm/include", f"-I{tinc}", f"-I{tinc / 'torch/csrc/api/include'}",
               "-DUSE_ROCM=1", "-D_GLIBCXX_USE_CXX11_ABI=1", "-Wno-deprecated-declarations"]
     jobs_list = []
+    # the shape-generic kernels also serve true-f32 runs: precise exp / log / division, no
+    # reassociation (their f32 results are compared at f32 rounding level)
+    precise = [f for f in kflags if f != "-ffast-math"]
     for src in sorted((CSRC / "kernels").glob("*.hip")):
-        jobs_list.append((kflags, src, OBJ / "kernels" / (src.stem + ".o")))
+        fl = precise if src.stem in PRECISE_KERNELS else kflags
+        jobs_list.append((fl, src, OBJ / "kernels" / (src.stem + ".o")))
     for src in sorted((CSRC / "bindings").glob("*.cpp")):
         jobs_list.append((bflags, src, OBJ / "bindings" / (src.stem + ".o")))
     objs, rebuilt = [], False

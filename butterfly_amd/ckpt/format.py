@@ -90,7 +90,33 @@ def save(model, path: str | os.PathLike, rank: int = 0, world: int = 1, comm=Non
         comm.barrier()
 
 
+def _plain_manifest(root: Path) -> dict:
+    """Manifest of a plain model folder (config.json + *.safetensors holding whole tensors under
+    the model's logical names), built from the safetensors headers."""
+    cfg = ModelConfig.from_model_dir(root)
+    tensors: dict = {}
+    dts = set()
+    for f in sorted(root.glob("*.safetensors")):
+        with safe_open(str(f), framework="pt", device="cpu") as fh:
+            for k in fh.keys():
+                sl = fh.get_slice(k)
+                shape = list(sl.get_shape())
+                dt = {"BF16": "bf16", "F32": "f32", "F16": "f16"}.get(sl.get_dtype())
+                if dt is None:
+                    continue
+                dts.add(dt)
+                tensors[k] = {"shape": shape, "dtype": dt, "shards": [
+                    {"file": f.name, "split_dim": None, "offset": 0, "length": shape[0] if shape else 1}]}
+    if not tensors:
+        raise FileNotFoundError(f"no *.safetensors in {root}")
+    return {"format": FORMAT, "version": VERSION, "model": cfg.to_dict(), "plan": {},
+            "dtype": "bf16" if "bf16" in dts else sorted(dts)[0], "tensors": tensors}
+
+
 def read_manifest(path: str | os.PathLike) -> dict:
+    root = Path(path)
+    if not (root / "manifest.json").exists() and (root / "config.json").exists():
+        return _plain_manifest(root)
     m = json.loads((Path(path) / "manifest.json").read_text())
     if m.get("format") != FORMAT:
         raise ValueError(f"{path} is not a {FORMAT} checkpoint")
@@ -167,6 +193,8 @@ def load_into(model, path: str | os.PathLike, strict: bool = True) -> list:
             raise ValueError(f"checkpoint {k}={getattr(saved_cfg, k)} != model {getattr(c, k)}")
     reader = _Reader(root)
     missing = []
+    if hasattr(model, "set_decay_ranks"):   # sizes that only tensor shapes give
+        model.set_decay_ranks({k: v["shape"] for k, v in manifest["tensors"].items()})
     with torch.no_grad():
         for lp in model.logical_params():
             if lp.split_dim is not None and lp.length == 0:

@@ -104,6 +104,76 @@ def cmd_generate(a) -> int:
     return 0
 
 
+def cmd_trace_run(a) -> int:
+    """Replay a recorded schedule through the engine, step by step, and write the logits it asks
+    for. Standard input: one JSON object per line,
+        {"step": n, "entries": [{"id": ..., "tokens": [...], "want": [...]}], "end": [ids]}
+    `entries`: the requests that run in this step with their next tokens and the offsets among
+    them whose logits are wanted; `end`: requests finished after the step (cache pages and state
+    slot are returned). For a step with wanted rows <out>/<step>.f32 holds them as little-endian
+    f32 [rows, vocab]; after every step a line "done <step>" is printed. Nothing is sampled."""
+    import numpy as np
+    import torch
+
+    from .ckpt import load_into, model_config
+    from .config import EngineConfig
+    from .engine.engine import LLMEngine
+    from .models import build_model
+
+    want32 = a.dtype in ("float32", "fp32")
+    dev = os.environ.get("BFLY_TRACE_DEVICE") or ("cuda" if torch.cuda.is_available() else None)
+    if dev is None:
+        print("trace-run needs a GPU (BFLY_TRACE_DEVICE=cpu runs the reference ops instead)", file=sys.stderr)
+        return 4
+    device = torch.device(dev)
+    if device.type == "cuda":
+        from . import ops
+
+        if not ops.load_library():        # fresh checkout: compile the kernel library once
+            from . import _build
+
+            _build.build_all(verbose=False)
+            ops.require_library()
+    cfg = model_config(a.model)
+    model = build_model(cfg, device=device, dtype=torch.float32 if (want32 or device.type == "cpu") else torch.bfloat16)
+    load_into(model, a.model)
+    bs = 32
+    cap = (max(a.max_tokens, bs) + bs - 1) // bs * bs
+    ecfg = EngineConfig(max_batch=a.max_requests, max_seq_len=cap, max_prefill_tokens=cap, block_size=bs,
+                        kv_cache_tokens=cap, use_graphs=not a.no_graphs, dtype="fp32" if want32 else "bf16",
+                        mixed_prefill=True, prefix_caching=False, async_decode=False,
+                        graph_batch_sizes=sorted({1, 2, 4, a.max_requests}))
+    eng = LLMEngine(cfg, engine_cfg=ecfg, model=model, device=device)
+    os.makedirs(a.out, exist_ok=True)
+    rid_of: dict = {}
+    next_rid = 0
+    for line in sys.stdin:
+        line = line.strip()
+        if not line:
+            continue
+        st = json.loads(line)
+        entries = []
+        for e in st.get("entries", []):
+            if e["id"] not in rid_of:
+                rid_of[e["id"]] = next_rid
+                next_rid += 1
+            rid = rid_of[e["id"]]
+            entries.append((rid, e["tokens"], e.get("want", [])))
+        end = [rid_of[i] for i in st.get("end", []) if i in rid_of]
+        logits = eng.replay_step(entries, end)
+        if logits is not None:
+            arr = logits.detach().to("cpu", torch.float32).contiguous().numpy().astype("<f4", copy=False)
+            tmp = os.path.join(a.out, f".{st['step']}.part")
+            with open(tmp, "wb") as f:
+                f.write(np.ascontiguousarray(arr).tobytes())
+            os.replace(tmp, os.path.join(a.out, f"{st['step']}.f32"))
+        for i in st.get("end", []):
+            rid_of.pop(i, None)
+        print(f"done {st['step']}", flush=True)
+    eng.close()
+    return 0
+
+
 def cmd_serve(a) -> int:
     from .api import LLM
     from .config import EngineConfig
@@ -230,6 +300,15 @@ def main(argv=None) -> int:
     c.add_argument("--gpus", type=int, default=1)
     c.add_argument("--strategy", default="auto")
     c.set_defaults(fn=cmd_ckpt)
+    t = sub.add_parser("trace-run", help="replay a recorded schedule (JSON steps on stdin) and write logits")
+    t.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    t.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    t.add_argument("--out", required=True, help="folder for <step>.f32")
+    t.add_argument("--max-tokens", type=int, required=True,
+                   help="tokens the live requests hold at most (the cache pool is made for this many)")
+    t.add_argument("--max-requests", type=int, default=4, help="live requests at most (state slots)")
+    t.add_argument("--no-graphs", action="store_true")
+    t.set_defaults(fn=cmd_trace_run)
     i = sub.add_parser("info")
     i.set_defaults(fn=cmd_info)
     a = ap.parse_args(argv)

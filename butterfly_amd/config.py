@@ -16,7 +16,7 @@ from typing import Any, Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str                       # "llama" | "gpt2" | "mixtral"
+    arch: str                       # "llama" | "gpt2" | "mixtral" | "nesizen"
     vocab_size: int
     hidden_size: int
     intermediate_size: int
@@ -36,6 +36,10 @@ class ModelConfig:
     num_experts: int = 0            # > 0: MoE FFN
     experts_per_token: int = 0
     init_std: float = 0.02
+    # heterogeneous stacks (arch "nesizen"): one normalised spec per layer (layer_spec below);
+    # the flat fields above then hold the largest value over the layers (workspace sizing)
+    layer_specs: Optional[list] = None
+    residual_streams: int = 1       # > 1: hyper-connections (parallel residual streams)
 
     # ---- derived quantities ------------------------------------------------------------
     @property
@@ -54,6 +58,8 @@ class ModelConfig:
         return (self.vocab_size + multiple - 1) // multiple * multiple
 
     def layer_params(self) -> int:
+        if self.layer_specs:
+            return sum(layer_spec_params(self.hidden_size, sp) for sp in self.layer_specs) // len(self.layer_specs)
         h, f = self.hidden_size, self.intermediate_size
         attn = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
         mlp = (3 if self.act == "silu" else 2) * h * f
@@ -81,6 +87,9 @@ class ModelConfig:
         return self.param_count() - self.num_layers * (self.layer_params() - per_layer)
 
     def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        if self.layer_specs:
+            return sum(sp["kv_heads"] * (sp["dim"] + sp["vdim"]) * dtype_bytes for sp in self.layer_specs
+                       if sp["type"] == "attention" and sp["kv_from"] is None)
         return 2 * self.num_layers * self.kv_size * dtype_bytes
 
     # ---- (de)serialisation -------------------------------------------------------------
@@ -99,6 +108,40 @@ class ModelConfig:
         d = dict(PRESETS[name])
         d.update(overrides)
         return cls(name=name, **d)
+
+    @classmethod
+    def from_nesizen(cls, js: dict, name: str = "nesizen") -> "ModelConfig":
+        """Map a Nesizen config.json ("architecture": "Nesizen") to ModelConfig. Every size and
+        every per-layer constant is taken from the file; layers may differ from one another."""
+        specs = [layer_spec(i, L) for i, L in enumerate(js["layers"])]
+        for sp in specs:
+            j = sp["kv_from"]
+            if j is not None:
+                o = specs[j] if 0 <= j < sp["index"] else None
+                if o is None or o["type"] != "attention" or o["kv_from"] is not None:
+                    raise ValueError(f"layer {sp['index']}: kv_from must name an earlier attention layer with its own keys")
+                if (o["kv_heads"], o["dim"], o["vdim"]) != (sp["kv_heads"], sp["dim"], sp["vdim"]):
+                    raise ValueError(f"layer {sp['index']}: key/value shape differs from layer {j}")
+        mx = lambda key: max([sp.get(key) or 0 for sp in specs] + [0])  # noqa: E731
+        moe = [sp["ffn"] for sp in specs if sp["ffn"] and sp["ffn"]["kind"] == "moe"]
+        return cls(name=name, arch="nesizen", vocab_size=int(js["vocab"]), hidden_size=int(js["width"]),
+                   intermediate_size=max([sp["ffn"]["ff"] for sp in specs if sp["ffn"]] + [0]),
+                   num_layers=len(specs), num_heads=mx("heads"), num_kv_heads=max(mx("kv_heads"), 1),
+                   head_dim=max(mx("dim"), mx("vdim")), max_position=1 << 30, norm_eps=float(js["norm"]["eps"]),
+                   norm="rms", act="relu2", pos_emb="rope", tie_embeddings=False,
+                   num_experts=max([m["experts"] for m in moe] + [0]),
+                   experts_per_token=max([m["top"] for m in moe] + [0]),
+                   layer_specs=specs, residual_streams=int(js.get("streams", 1)))
+
+    @classmethod
+    def from_model_dir(cls, path, name: Optional[str] = None) -> "ModelConfig":
+        """config.json of a model folder -> ModelConfig; the "architecture" / "model_type" key
+        chooses the family."""
+        js = json.loads((Path(path) / "config.json").read_text())
+        name = name or Path(path).name
+        if str(js.get("architecture", "")).lower() == "nesizen":
+            return cls.from_nesizen(js, name=name)
+        return cls.from_hf(js, name=name)
 
     @classmethod
     def from_hf(cls, hf: dict, name: str = "hf") -> "ModelConfig":
@@ -132,6 +175,54 @@ class ModelConfig:
                    tie_embeddings=hf.get("tie_word_embeddings", False),
                    num_experts=hf.get("num_local_experts", 0),
                    experts_per_token=hf.get("num_experts_per_tok", 0))
+
+
+def layer_spec(index: int, L: dict) -> dict:
+    """One layer of a heterogeneous stack, normalised to flat keys. `type` "attention": windowed
+    softmax attention (heads, kv_heads, dim, vdim, rot_dims, rot_base, scale, window, keep_first,
+    kv_from); "gla": gated linear attention (heads, dim, vdim, tau). `ffn`: None, or kind
+    "dense" (ff) / "moe" (ff, limit, experts, top)."""
+    m, t = L["mixer"], L["type"]
+    sp = {"index": index, "type": t, "heads": int(m["heads"]), "dim": int(m["dim"]), "vdim": int(m["vdim"]),
+          "kv_from": None, "kv_heads": 0}
+    if t == "attention":
+        sp.update(kv_heads=int(m.get("kv_heads", m["heads"])), rot_dims=int(m["rot"]["dims"]),
+                  rot_base=float(m["rot"]["base"]), scale=float(m["scale"]), window=int(m["mask"]["size"]),
+                  keep_first=int(m["mask"].get("keep_first", 0)),
+                  kv_from=None if m.get("kv_from") is None else int(m["kv_from"]))
+        if sp["heads"] % sp["kv_heads"] or sp["rot_dims"] % 2 or sp["rot_dims"] > sp["dim"]:
+            raise ValueError(f"layer {index}: bad attention sizes")
+    elif t == "gla":
+        sp.update(tau=float(m["tau"]))
+    else:
+        raise ValueError(f"layer {index}: unknown mixer type {t!r}")
+    f = L.get("mlp")
+    if f is None:
+        sp["ffn"] = None
+    elif f["kind"] == "dense":
+        sp["ffn"] = {"kind": "dense", "ff": int(f["ff"])}
+    elif f["kind"] == "moe":
+        sp["ffn"] = {"kind": "moe", "ff": int(f["expert"]["ff"]), "limit": float(f["expert"]["limit"]),
+                     "experts": int(f["router"]["experts"]), "top": int(f["router"]["top"])}
+        if not 1 <= sp["ffn"]["top"] <= sp["ffn"]["experts"]:
+            raise ValueError(f"layer {index}: top must be in 1..experts")
+    else:
+        raise ValueError(f"layer {index}: unknown feed-forward kind {f['kind']!r}")
+    return sp
+
+
+def layer_spec_params(h: int, sp: dict) -> int:
+    H, D, Dv = sp["heads"], sp["dim"], sp["vdim"]
+    if sp["type"] == "attention":
+        n = h * H * D + H * Dv * h + H
+        if sp["kv_from"] is None:
+            n += h * sp["kv_heads"] * (D + Dv)
+    else:
+        n = h * H * (2 * D + 2 * Dv) + H * Dv * h + Dv
+    f = sp["ffn"]
+    if f:
+        n += 2 * h * f["ff"] if f["kind"] == "dense" else f["experts"] * (3 * h * f["ff"] + h)
+    return n + 2 * h
 
 
 PRESETS: dict[str, dict[str, Any]] = {

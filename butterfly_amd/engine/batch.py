@@ -39,6 +39,9 @@ class ForwardBatch:
     cu_fresh: Optional[torch.Tensor] = None
     max_fresh: int = 0
     max_paged: int = 0
+    # recurrent-state slot of every sequence of the step (decode rows' sequences, then the prompt
+    # chunks'), for models with per-sequence state (int32; -1: padding row, no state)
+    state_slots: Optional[torch.Tensor] = None
 
     @property
     def num_tokens(self) -> int:
@@ -57,7 +60,7 @@ class ForwardBatch:
                             mv(self.ctx_lens), self.max_ctx, mv(self.logits_idx), self.ep_tokens,
                             self.ep_alltoall, self.cp, self.num_decode, self.prefix_lens,
                             mv(self.prefix_cu), mv(self.prefix_tables), self.split_seqs, self.split_rows,
-                            mv(self.cu_fresh), self.max_fresh, self.max_paged)
+                            mv(self.cu_fresh), self.max_fresh, self.max_paged, mv(self.state_slots))
 
 
 def make_prefill_batch(prompts: list[list[int]], slots: list[list[int]], device="cpu",

@@ -119,7 +119,10 @@ class LLMEngine:
         a, b = stage_layers[coord.pp]
         shard = Shard(tp_rank=coord.tp, tp_size=mesh.tp, layer_start=a, layer_end=b,
                       ep_rank=coord.dp if mesh.ep > 1 else 0, ep_size=mesh.ep)
-        dtype = torch.bfloat16 if self.device.type == "cuda" else torch.float32
+        # EngineConfig.dtype "fp32": true 32-bit weights, activations and caches (models whose
+        # kernels have an f32 form; the bf16-only families refuse it on the GPU)
+        want32 = str(engine_cfg.dtype).lower() in ("fp32", "float32", "f32")
+        dtype = torch.float32 if (self.device.type != "cuda" or want32) else torch.bfloat16
         self.model = model or build_model(cfg, shard, device=self.device, dtype=dtype, comm=self.comm)
         if model is None:
             self.model.init_random(engine_cfg.seed)
@@ -146,7 +149,9 @@ class LLMEngine:
             if room > 0:
                 kinds = [k.strip() for k in flags.get("BFLY_PACKED_KINDS").split(",") if k.strip()]
                 self.model.pack_decode_weights(budget_bytes=room, kinds=kinds)
-        self.kv = KVCache(self.model, nblocks, bs, self.kv_dtype)
+        # models with recurrent layers: one state slot per sequence the batch can hold
+        self.kv = KVCache(self.model, nblocks, bs, self.kv_dtype,
+                          state_slots=engine_cfg.max_batch if getattr(self.model, "has_state", False) else 0)
         native = __import__("butterfly_amd._native_loader", fromlist=["native"]).native()
         # pipeline parallelism without per-step fill/drain: pp request groups in flight
         # (engine/pipeline.py); EP layouts keep the synchronous path (EP collectives span DP ranks)
@@ -162,7 +167,10 @@ class LLMEngine:
         # agree per step on the padded row count and on whether any of them runs prompt rows
         # (which switches every peer's MoE layer to the variable exchange): _ep_agree
         self.mixed = bool(engine_cfg.mixed_prefill) and (mesh.pp == 1 or self.async_pp)
-        self.prefix_cache = self.mixed and bool(engine_cfg.prefix_caching)
+        # (cached prefix pages hold keys and values, not a recurrent state: off for such models)
+        self.prefix_cache = self.mixed and bool(engine_cfg.prefix_caching) and not self.kv.state_slots
+        if getattr(self.model, "paged_prefill_only", False) and not self.mixed:
+            raise ValueError(f"{cfg.arch} models need mixed scheduling (EngineConfig.mixed_prefill)")
         if self.async_pp:
             self.scheduler = GroupedScheduler(native, self.kv.manager, mesh.pp, engine_cfg.max_batch,
                                               engine_cfg.max_prefill_tokens, self.mixed, self.prefix_cache)
@@ -976,6 +984,67 @@ class LLMEngine:
                 torch.empty(0, dtype=torch.int32, device=self.device)
 
         self._execute(self._ops(1, native_dec), recv, run, send, sample)
+
+    # ------------------------------------------------------------------------------------
+    # replay of a recorded schedule (runtime/scheduler.h schedule_script)
+    def replay_step(self, entries: list, end: Optional[list] = None) -> Optional[torch.Tensor]:
+        """One step of a recorded schedule: `entries` = [(rid, next tokens, wanted offsets)] for
+        the requests that run in this step, `end` = requests that are finished after it (their
+        pages and state slot are returned). A request is admitted at its first entry; one token
+        of a request that already holds tokens runs as a decode row, anything else as a prompt
+        chunk over its cached prefix, all in one batch through the same runner, caches and kernels
+        as generation. Nothing is sampled: returns the logits [wanted rows, vocab] f32 in the
+        order of the entries and their wanted offsets (None if nothing is wanted). Synchronous
+        single-stage engines only (EngineConfig.async_decode = False)."""
+        if self.async_pp or self.mesh.world_size != 1:
+            raise RuntimeError("replay_step needs a synchronous single-rank engine (async_decode=False)")
+        sched = []
+        for rid, toks, _ in entries:
+            req = self.requests.get(rid)
+            if req is None:
+                req = self.requests[rid] = Request(rid, [], SamplingParams(max_tokens=1), arrival=time.perf_counter())
+            req.prompt.extend(int(t) for t in toks)
+            sched.append((rid, len(toks)))
+        logits = None
+        if sched:
+            plan = self.scheduler.schedule_script(sched)
+            if plan.cow:
+                self.kv.copy_blocks(list(plan.cow))
+            rows = self._plan_rows(plan)
+            want = [rows[rid] + int(o) for rid, _, offs in entries for o in offs]
+            if plan.kind == 2 and self.runner.use_graphs:
+                last = [self.requests[r].prompt[-1] for r in plan.seq_ids]
+                out = self.runner.run_decode(self.runner.decode_inputs(plan, last))
+                if want:
+                    logits = out[torch.tensor(want, dtype=torch.int64, device=out.device)]
+            else:
+                fb, _ = self.runner.mixed_batch(plan, lambda r: self.requests[r].prompt)
+                if not want:
+                    want = [0]            # the step still runs (it fills caches and state)
+                    fb.logits_idx = torch.tensor(want, dtype=torch.int64).to(self.device)
+                    self.runner.run(fb)
+                else:
+                    fb.logits_idx = torch.tensor(want, dtype=torch.int64).to(self.device)
+                    logits = self.runner.run(fb)
+            if logits is not None:
+                logits = logits[:, :self.cfg.vocab_size].float()
+        for rid in end or []:
+            self.scheduler.finish(rid)
+            self.requests.pop(rid, None)
+        self.steps_done += 1
+        return logits
+
+    @staticmethod
+    def _plan_rows(plan) -> dict:
+        """First batch row of every sequence of a mixed-layout plan (decode rows, then chunks)."""
+        nd = plan.num_decode
+        sids = list(plan.seq_ids)
+        rows = {sid: i for i, sid in enumerate(sids[:nd])}
+        at = nd
+        for sid, n in zip(sids[nd:], plan.prefill_lens):
+            rows[sid] = at
+            at += int(n)
+        return rows
 
     def close(self) -> dict:
         """Release the engine's device resources in dependency order: captured graphs first

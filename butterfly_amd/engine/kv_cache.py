@@ -34,20 +34,28 @@ def device_kv_budget(device: torch.device, utilization: float, reserve_bytes: in
 
 
 class KVCache:
-    def __init__(self, model, num_blocks: int, block_size: int, dtype: Optional[torch.dtype] = None):
+    def __init__(self, model, num_blocks: int, block_size: int, dtype: Optional[torch.dtype] = None,
+                 state_slots: int = 0):
+        """`state_slots` > 0 (models with recurrent layers, `model.has_state`): a pool of that many
+        per-sequence state rows beside the pages (model.allocate_state: one f32 tensor per recurrent
+        layer); the block manager gives every live sequence one slot and takes it back with its
+        pages."""
         self.block_size = block_size
         self.num_blocks = num_blocks
         self.layers = model.allocate_kv_cache(num_blocks, block_size, dtype)
         self.dtype = self.layers[0][0].dtype if self.layers else dtype
+        self.state_slots = state_slots if getattr(model, "has_state", False) else 0
+        self.state = model.allocate_state(self.state_slots) if self.state_slots else []
         native = _native_loader.native()
-        self.manager = native.KVBlockManager(num_blocks, block_size)
+        self.manager = native.KVBlockManager(num_blocks, block_size, self.state_slots)
 
     @property
     def capacity_tokens(self) -> int:
         return self.num_blocks * self.block_size
 
     def bytes(self) -> int:
-        return sum(k.numel() * k.element_size() + v.numel() * v.element_size() for k, v in self.layers)
+        return sum(k.numel() * k.element_size() + v.numel() * v.element_size() for k, v in self.layers) + \
+            sum(t.numel() * t.element_size() for t in self.state)
 
     def copy_blocks(self, pairs: list) -> None:
         """Copy-on-write page copies (src -> dst) before a step that writes to a forked page."""

@@ -64,9 +64,11 @@ class _DecodeGraph:
         self.off_s = (self.off_t + b + 1) // 2 * 2        # seeds: 8-byte aligned int32 offset
         # initial state built on the host and copied once: padding rows have no cache slot (-1)
         # and context 1 (no torch fill kernels on the device)
-        init = torch.zeros(self.off_s + 2 * b, dtype=torch.int32)
+        self.off_st = self.off_s + 2 * b                  # recurrent-state slots (-1: none)
+        init = torch.zeros(self.off_st + b, dtype=torch.int32)
         init[2 * b:3 * b] = -1
         init[3 * b:4 * b] = 1
+        init[self.off_st:] = -1
         self.inbuf = init.to(device)
         self.input_ids = self.inbuf[0:b]
         self.positions = self.inbuf[b:2 * b]
@@ -75,6 +77,7 @@ class _DecodeGraph:
         self.block_tables = self.inbuf[4 * b:self.off_t].view(b, max_blocks)
         self.temps = self.inbuf[self.off_t:self.off_t + b].view(torch.float32)
         self.seeds = self.inbuf[self.off_s:self.off_s + 2 * b].view(torch.int64)
+        self.state_slots = self.inbuf[self.off_st:self.off_st + b]
         self.ids: Optional[torch.Tensor] = None     # sampled in the graph (last stage)
         pin = torch.cuda.is_available() and torch.device(device).type == "cuda"
         self.host = [torch.zeros(self.inbuf.numel(), dtype=torch.int32, pin_memory=pin) for _ in range(2)]
@@ -97,6 +100,10 @@ class ModelRunner:
         self.device = model.device
         self.max_seq_len = max_seq_len
         self.block_size = kv_cache.block_size
+        # models with per-sequence recurrent state get every step's state slots; models whose
+        # prompt chunks always read keys through the block tables get the tables of fresh prompts too
+        self.stateful = bool(getattr(kv_cache, "state_slots", 0))
+        self.paged_only = bool(getattr(model, "paged_prefill_only", False))
         self.max_blocks = (max_seq_len + self.block_size - 1) // self.block_size
         self.use_graphs = use_graphs and self.device.type == "cuda" and \
             os.environ.get("BFLY_DISABLE_GRAPHS", "0") != "1"
@@ -183,7 +190,7 @@ class ModelRunner:
             self.kv.manager.fill_decode_tables(dec, self._tables_host[:nd], self._ctx_host[:nd])
             bt = torch.from_numpy(self._tables_host[:nd].copy()).to(dev, non_blocking=True)
             ctx = torch.from_numpy(self._ctx_host[:nd].copy()).to(dev, non_blocking=True)
-        if any(prefix):
+        if any(prefix) or (self.paged_only and chunk_sids):
             pc = [0]
             for p in prefix:
                 pc.append(pc[-1] + p)
@@ -201,7 +208,8 @@ class ModelRunner:
                           block_tables=bt, ctx_lens=ctx, max_ctx=self.max_seq_len,
                           logits_idx=torch.tensor(rows, dtype=torch.int64).to(dev, non_blocking=True),
                           num_decode=nd, prefix_lens=prefix if any(prefix) else None, prefix_cu=pre_cu,
-                          prefix_tables=pre_tab)
+                          prefix_tables=pre_tab,
+                          state_slots=t32(self.kv.manager.state_slots_of(dec + chunk_sids)) if self.stateful else None)
         # continuation chunks first, fresh prompts after them (the scheduler's order when it
         # resumes a partly prefilled prompt): only the continuations need the paged pass
         s1 = next((j for j, p in enumerate(prefix) if p == 0), len(prefix))
@@ -215,17 +223,21 @@ class ModelRunner:
         B = len(plan.seq_ids)
         self.kv.manager.fill_decode_tables(list(plan.seq_ids), self._tables_host[:B], self._ctx_host[:B])
         ids = last_tokens if isinstance(last_tokens, torch.Tensor) else np.asarray(last_tokens, dtype=np.int32)
-        return dict(ids=ids,
-                    pos=np.asarray(plan.decode_positions, dtype=np.int32),
-                    slots=np.asarray(plan.decode_slots, dtype=np.int32),
-                    tables=self._tables_host[:B], ctx=self._ctx_host[:B])
+        inp = dict(ids=ids,
+                   pos=np.asarray(plan.decode_positions, dtype=np.int32),
+                   slots=np.asarray(plan.decode_slots, dtype=np.int32),
+                   tables=self._tables_host[:B], ctx=self._ctx_host[:B])
+        if self.stateful:
+            inp["state"] = np.asarray(self.kv.manager.state_slots_of(list(plan.seq_ids)), dtype=np.int32)
+        return inp
 
     def decode_batch(self, inp: dict, ep_tokens: int = 0) -> ForwardBatch:
         dev = self.device
         t = lambda a: _to_dev(a, dev)  # noqa: E731
         return ForwardBatch(input_ids=t(inp["ids"]), positions=t(inp["pos"]), slots=t(inp["slots"]),
                             is_prefill=False, block_tables=t(inp["tables"]), ctx_lens=t(inp["ctx"]),
-                            max_ctx=self.max_seq_len, logits_idx=None, ep_tokens=ep_tokens)
+                            max_ctx=self.max_seq_len, logits_idx=None, ep_tokens=ep_tokens,
+                            state_slots=t(inp["state"]) if inp.get("state") is not None else None)
 
     # ------------------------------------------------------------------------------------
     def run(self, fb: ForwardBatch, hidden_in=None):
@@ -372,6 +384,9 @@ class ModelRunner:
         ht[B:] = 0.0
         hs[:B] = 0 if sd is None else sd
         hs[B:] = 0
+        st = inp.get("state")
+        h[g.off_st:g.off_st + B] = -1 if st is None else st
+        h[g.off_st + B:g.off_st + b] = -1
         start = b if ids_dev else 0
         g.inbuf[start:].copy_(g.host[k][start:], non_blocking=True)
         if self.device.type == "cuda":
@@ -388,7 +403,8 @@ class ModelRunner:
     def _graph_batch(self, g: _DecodeGraph) -> ForwardBatch:
         return ForwardBatch(input_ids=g.input_ids, positions=g.positions, slots=g.slots,
                             is_prefill=False, block_tables=g.block_tables, ctx_lens=g.ctx_lens,
-                            max_ctx=self.max_seq_len, logits_idx=None, ep_tokens=g.bucket)
+                            max_ctx=self.max_seq_len, logits_idx=None, ep_tokens=g.bucket,
+                            state_slots=g.state_slots if self.stateful else None)
 
     def _capture(self, bucket: int, register: bool = True) -> _DecodeGraph:
         m = self.model

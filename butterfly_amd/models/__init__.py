@@ -1,6 +1,8 @@
-"""Model families: Llama-3 (8B/70B), Mixtral 8x7B (MoE), GPT-2 — one shard-aware decoder."""
+"""Model families: Llama-3 (8B/70B), Mixtral 8x7B (MoE), GPT-2 — one shard-aware decoder — and
+Nesizen, a heterogeneous stack of attention / gated-linear-attention layers (models/nesizen.py)."""
 from .shard import LocalDims, Shard, local_dims  # noqa: F401
 from .transformer import LogicalParam, TransformerLM  # noqa: F401
+from .nesizen import NesizenLM  # noqa: F401
 
 
 class LlamaForCausalLM(TransformerLM):
@@ -15,7 +17,8 @@ class GPT2LMHeadModel(TransformerLM):
     """GPT-2 (learned positions, LayerNorm, GELU MLP with biases, tied embeddings)."""
 
 
-_ARCH = {"llama": LlamaForCausalLM, "mixtral": MixtralForCausalLM, "gpt2": GPT2LMHeadModel}
+_ARCH = {"llama": LlamaForCausalLM, "mixtral": MixtralForCausalLM, "gpt2": GPT2LMHeadModel,
+         "nesizen": NesizenLM}
 
 
 def build_model(cfg, shard=None, device="cpu", dtype=None, comm=None):

@@ -714,3 +714,149 @@ def moe_gate_scale_(h, gates, e0: int, num_local: int):
         return ref.moe_gate_scale(h, gates, e0, num_local)
     torch.ops.bfly.moe_gate_scale(h, gates, e0, num_local)
     return h
+
+
+# ---------------------------------------------------------------------------------------
+# Shape-generic ops (csrc/kernels/gemm_any.hip, hyper.hip, mixers.hip): bf16 or f32 tensors
+# ---------------------------------------------------------------------------------------
+ACTS = {"none": 0, "relu2": 1}
+
+
+def _mfma_gemm_ok(x, w, out_dtype) -> bool:
+    """The MFMA GEMM family takes bf16 operands with K % 64 == 0, N % 128 == 0 and 16-byte rows."""
+    return (x.dtype == torch.bfloat16 and out_dtype in (None, torch.bfloat16) and w.shape[1] % 64 == 0
+            and w.shape[0] % 128 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and x.shape[0] > 0)
+
+
+def linear_act(x, w, bias=None, act: str = "none", out_dtype=None):
+    """y = act(x w^T + bias) for any shape, bf16 or f32 (`out_dtype` f32: keep the f32
+    accumulator). bf16 shapes the MFMA GEMMs tile go to them (the activation as a pass over the
+    result); every other shape, and f32, runs the generic tile kernel."""
+    if not _gpu(x):
+        return ref.linear_act(x, w, bias, act, out_dtype)
+    if _mfma_gemm_ok(x, w, out_dtype):
+        y = linear(x, w, bias=bias)
+        if act == "relu2":
+            torch.ops.bfly.relu2_(y)
+        return y
+    out = _empty(x.shape[0], w.shape[0], dtype=out_dtype or x.dtype, device=x.device)
+    torch.ops.bfly.gemm_any(x, w, bias, ACTS[act], out)
+    return out
+
+
+def embed_norm_streams(ids, table, norm_w, eps: float, offset: float, streams: int):
+    """Token embedding, RMS norm with weight (w + offset), copied into `streams` parallel
+    residual streams: xs [T, streams, W] f32."""
+    if not _gpu(table):
+        return ref.embed_norm_streams(ids, table, norm_w, eps, offset, streams)
+    xs = _empty(ids.numel(), streams, table.shape[1], dtype=torch.float32, device=table.device)
+    torch.ops.bfly.embed_norm_streams(ids, table, norm_w, eps, offset, xs)
+    return xs
+
+
+def hc_pre(xs, w_in, norm_w, eps: float, offset: float, out_dtype):
+    """A sublayer's input: the streams mixed by w_in [S], RMS-normed with weight (w + offset)."""
+    if not _gpu(xs):
+        return ref.hc_pre(xs, w_in, norm_w, eps, offset, out_dtype)
+    out = _empty(xs.shape[0], xs.shape[2], dtype=out_dtype, device=xs.device)
+    torch.ops.bfly.hc_pre(xs, w_in, norm_w, eps, offset, out)
+    return out
+
+
+def hc_post_(xs, y, mix, w_out):
+    """xs[:, r] <- sum_s mix[s, r] xs[:, s] + w_out[r] y, in place (all streams from the old ones)."""
+    if not _gpu(xs):
+        return ref.hc_post_(xs, y, mix, w_out)
+    torch.ops.bfly.hc_post(xs, y, mix, w_out)
+    return xs
+
+
+def hc_final(xs, norm_w, eps: float, offset: float, idx, out_dtype):
+    """Sum of the streams of rows `idx` (None: all), RMS-normed with weight (w + offset)."""
+    if not _gpu(xs):
+        return ref.hc_final(xs, norm_w, eps, offset, idx, out_dtype)
+    R = xs.shape[0] if idx is None else idx.numel()
+    out = _empty(R, xs.shape[2], dtype=out_dtype, device=xs.device)
+    torch.ops.bfly.hc_final(xs, norm_w, eps, offset, idx, out)
+    return out
+
+
+def rope_partial_kv(q, k, v, positions, inv_freq, slots=None, k_cache=None, v_cache=None):
+    """Interleaved-pair rotary on the first 2 * len(inv_freq) dims of the q [T, H, D] and
+    k [T, G, D] heads, in place, and the append of k, v [T, G, Dv] to the paged caches
+    K [blocks, G, BS, D], V [blocks, G, BS, Dv]. k None: q only."""
+    if not _gpu(q):
+        return ref.rope_partial_kv(q, k, v, positions, inv_freq, slots, k_cache, v_cache)
+    torch.ops.bfly.rope_partial_kv(q, k, v, positions, inv_freq, slots, k_cache, v_cache)
+    return q
+
+
+def row_seq(row_cu, T: int):
+    """Row -> sequence map of a packed step (rows outside every sequence: -1); GPU only."""
+    out = _empty(T, dtype=torch.int32, device=row_cu.device)
+    torch.ops.bfly.row_seq(row_cu, out)
+    return out
+
+
+def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale: float, window: int, keep_first: int,
+                      sink, row_map=None, out=None):
+    """Windowed attention of packed rows over the paged cache with kept first positions and a
+    sink logit (mixers.hip attn_window_paged_kernel). `row_map`: ops.row_seq(row_cu, T), when the
+    caller already has it."""
+    if not _gpu(q):
+        return ref.attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, window, keep_first, sink, out)
+    if out is None:
+        out = _empty(q.shape[0], q.shape[1], v_cache.shape[3], dtype=q.dtype, device=q.device)
+    if row_map is None:
+        row_map = row_seq(row_cu, q.shape[0])
+    torch.ops.bfly.attn_window_paged(q, k_cache, v_cache, tables, row_map, positions, float(scale), int(window),
+                                     int(keep_first), sink, out)
+    return out
+
+
+def gla_scan(q, k, v, z, state, state_slots, row_cu, positions, tau: float, q_scale: float):
+    """Gated linear attention over packed rows with the state pooled in `state` [slots, H, D, Dv]
+    f32 (updated in place). Returns o [T, H, Dv] f32."""
+    if not _gpu(q):
+        return ref.gla_scan(q, k, v, z, state, state_slots, row_cu, positions, tau, q_scale)
+    o = _empty(q.shape[0], q.shape[1], v.shape[2], dtype=torch.float32, device=q.device)
+    torch.ops.bfly.gla_scan(q, k, v, z, state, state_slots, row_cu, positions, float(tau), float(q_scale), o)
+    return o
+
+
+def gla_out(o, g, norm_w, eps: float, out_dtype):
+    if not _gpu(o):
+        return ref.gla_out(o, g, norm_w, eps, out_dtype)
+    out = _empty(o.shape[0], o.shape[1] * o.shape[2], dtype=out_dtype, device=o.device)
+    torch.ops.bfly.gla_out(o, g, norm_w, eps, out)
+    return out
+
+
+def moe_route_scores(x, wr, top_k: int, scoring: str = "softmax", renorm: bool = True):
+    """Router with f32 logits -> (topk_ids [T, k] int32, topk_w [T, k] f32); scoring "softmax" |
+    "sigmoid", `renorm`: divide the chosen scores by their sum."""
+    if not _gpu(x):
+        return ref.moe_route_scores(x, wr, top_k, scoring, renorm)
+    T = x.shape[0]
+    ids = _empty(T, top_k, dtype=torch.int32, device=x.device)
+    w = _empty(T, top_k, dtype=torch.float32, device=x.device)
+    torch.ops.bfly.moe_route_scores(x, wr, top_k, {"softmax": 0, "sigmoid": 1}[scoring], bool(renorm), ids, w)
+    return ids, w
+
+
+def moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit: float, alpha: float):
+    """Routed experts with a clamped GLU, each run on (routing score * x); see
+    ops.reference.moe_glu_ffn. gate_up_w [E, 2F, H], down_w [E, H, F]."""
+    if not _gpu(x):
+        return ref.moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit, alpha)
+    T, H = x.shape
+    E, F = gate_up_w.shape[0], down_w.shape[2]
+    TK = T * topk_ids.shape[1]
+    mt = torch.ops.bfly.moe_sort_max_tiles(TK, E)
+    dev = x.device
+    work = _arena.get(dev, "moe_glu_work", TK + E + 1 + 2 * mt + 1, torch.int32)
+    hmid = _arena.get(dev, "moe_glu_mid", TK * F, x.dtype)
+    y = _arena.get(dev, "moe_glu_y", TK * H, torch.float32)
+    out = _empty(T, H, dtype=x.dtype, device=dev)
+    torch.ops.bfly.moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, float(limit), float(alpha), work, hmid, y, out)
+    return out

@@ -533,3 +533,167 @@ def ep_combine(back, slot):
     ext = torch.cat([back.float(), back.new_zeros(1, back.shape[1]).float()])
     idx = torch.where(slot >= 0, slot.long(), back.shape[0])
     return ext.index_select(0, idx.view(-1)).view(T, ep, -1).sum(1).to(back.dtype)
+
+
+# ---------------------------------------------------------------------------------------
+# Heterogeneous-stack mechanisms: offset-weight norms over parallel residual streams
+# (hyper-connections), partial interleaved rotary, windowed attention with kept first tokens
+# and a sink logit, gated linear attention with a per-sequence recurrent state, sigmoid-scored
+# MoE with clamped GLU experts. Caches of these mixers: K [blocks, G, BS, D], V [blocks, G, BS, Dv]
+# (both row layouts), recurrent state [slots, H, D, Dv] f32.
+# ---------------------------------------------------------------------------------------
+def linear_act(x, w, bias=None, act="none", out_dtype=None):
+    """y = act(x w^T + bias), f32 accumulation; act: none | relu2 (relu squared)."""
+    y = x.float() @ w.float().t()
+    if bias is not None:
+        y = y + bias.float()
+    if act == "relu2":
+        y = torch.relu(y).square()
+    elif act != "none":
+        raise ValueError(act)
+    return y.to(out_dtype or x.dtype)
+
+
+def _rms_offset(x, w, eps, offset):
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (w.float() + offset)
+
+
+def embed_norm_streams(ids, table, norm_w, eps, offset, streams):
+    x = _rms_offset(table[ids.long()].float(), norm_w, eps, offset)
+    return x.unsqueeze(1).repeat(1, streams, 1).contiguous()
+
+
+def hc_pre(xs, w_in, norm_w, eps, offset, out_dtype):
+    u = torch.einsum("s,tsw->tw", w_in.float(), xs)
+    return _rms_offset(u, norm_w, eps, offset).to(out_dtype)
+
+
+def hc_post_(xs, y, mix, w_out):
+    new = torch.einsum("sr,tsw->trw", mix.float(), xs) + w_out.float()[None, :, None] * y.float()[:, None, :]
+    xs.copy_(new)
+    return xs
+
+
+def hc_final(xs, norm_w, eps, offset, idx, out_dtype):
+    x = xs.sum(1) if idx is None else xs[idx.long()].sum(1)
+    return _rms_offset(x, norm_w, eps, offset).to(out_dtype)
+
+
+def rope_partial_kv(q, k, v, positions, inv_freq, slots, k_cache, v_cache):
+    """Rotate the first 2 * len(inv_freq) dims of every q / k head in place (pairs (2i, 2i+1),
+    angle position * inv_freq[i], f32) and append k, v rows to their cache slots."""
+    n = inv_freq.numel()
+    a = positions.float()[:, None] * inv_freq.float()[None]
+    c, s = torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
+    for t in (q, k):
+        if t is None or n == 0:
+            continue
+        tf = t.float()
+        u, w = tf[..., 0:2 * n:2], tf[..., 1:2 * n:2]
+        r = torch.stack([u * c - w * s, w * c + u * s], -1).flatten(-2)
+        t[..., :2 * n] = r.to(t.dtype)
+    if k is not None and slots is not None:
+        bs = k_cache.shape[2]
+        ok = slots >= 0
+        sl = slots[ok].long()
+        k_cache[sl // bs, :, sl % bs] = k[ok].to(k_cache.dtype)
+        v_cache[sl // bs, :, sl % bs] = v[ok].to(v_cache.dtype)
+    return q
+
+
+def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, window, keep_first, sink, out=None):
+    """Row r of sequence s (rows row_cu[s] .. row_cu[s+1]) at position p attends to the cached
+    keys j <= p of tables[s] with p - j < window or j < keep_first; the softmax denominator
+    also holds exp(sink[h])."""
+    T, H, D = q.shape
+    G, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    o = torch.zeros(T, H, Dv, dtype=torch.float32, device=q.device)
+    cu = row_cu.tolist()
+    pos = positions.tolist()
+    for s in range(len(cu) - 1):
+        if cu[s + 1] == cu[s]:
+            continue
+        pmax = max(pos[cu[s]:cu[s + 1]])
+        nb = pmax // bs + 1
+        blk = tables[s, :nb].long()
+        K = k_cache[blk].float().permute(1, 0, 2, 3).reshape(G, nb * bs, D)
+        V = v_cache[blk].float().permute(1, 0, 2, 3).reshape(G, nb * bs, Dv)
+        j = torch.arange(nb * bs, device=q.device)[None, :]
+        p = positions[cu[s]:cu[s + 1]].long()[:, None]
+        ok = (j <= p) & ((p - j < window) | (j < keep_first))
+        qs = q[cu[s]:cu[s + 1]].float()
+        for h in range(H):
+            g = h // (H // G)
+            sc = (qs[:, h] @ K[g].t()) * scale
+            sc = sc.masked_fill(~ok, float("-inf"))
+            sk = sink[h].float().expand(sc.shape[0], 1)
+            w = torch.softmax(torch.cat([sc, sk], 1), -1)[:, :-1]
+            o[cu[s]:cu[s + 1], h] = w @ V[g]
+    o = o.to(q.dtype)
+    if out is None:
+        return o
+    out.copy_(o)
+    return out
+
+
+def gla_scan(q, k, v, z, state, state_slots, row_cu, positions, tau, q_scale):
+    """Gated linear attention over packed rows: per sequence and head S <- diag(a_t) S + k_t v_t^T,
+    o_t = S^T (q_t * q_scale), a_t = sigmoid(z_t)^(1/tau), all f32. The state of sequence s is
+    read from state[state_slots[s]] unless its first row is at position 0 (then zero), and
+    written back after its last row. Returns o [T, H, Dv] f32."""
+    T, H, D = q.shape
+    Dv = v.shape[2]
+    o = torch.zeros(T, H, Dv, dtype=torch.float32, device=q.device)
+    la = F.logsigmoid(z.float().view(T, H, D)) / tau
+    a = torch.exp(la)
+    cu, pos, sl = row_cu.tolist(), positions.tolist(), state_slots.tolist()
+    qf, kf, vf = q.float() * q_scale, k.float(), v.float()
+    for s in range(len(cu) - 1):
+        if cu[s + 1] == cu[s] or sl[s] < 0:
+            continue
+        S = torch.zeros(H, D, Dv, dtype=torch.float32, device=q.device) if pos[cu[s]] == 0 else state[sl[s]].clone()
+        for t in range(cu[s], cu[s + 1]):
+            S = a[t][:, :, None] * S + kf[t][:, :, None] * vf[t][:, None, :]
+            o[t] = torch.einsum("hd,hdv->hv", qf[t], S)
+        state[sl[s]] = S
+    return o
+
+
+def gla_out(o, g, norm_w, eps, out_dtype):
+    """Per-head RMS norm of o [T, H, Dv] (weight [Dv] shared by the heads) times silu(g)."""
+    T, H, Dv = o.shape
+    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+    return (y.reshape(T, H * Dv) * F.silu(g.float())).to(out_dtype)
+
+
+def moe_route_scores(x, wr, top_k, scoring="softmax", renorm=True):
+    """Router in f32. scoring "softmax" | "sigmoid"; the top_k largest scores are chosen (ties:
+    lowest expert id); `renorm`: the chosen scores are divided by their sum."""
+    logits = x.float() @ wr.float().t()
+    sc = torch.softmax(logits, -1) if scoring == "softmax" else torch.sigmoid(logits)
+    w, ids = torch.topk(sc, top_k, -1)
+    if renorm:
+        w = w / w.sum(-1, keepdim=True)
+    return ids.to(torch.int32), w.contiguous()
+
+
+def moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit, alpha, out_dtype=None):
+    """Routed experts with clamped GLU: for every chosen (token, expert) the expert runs on
+    w * x: g = min(Wg h, limit), u = clamp(Wu h, -limit, limit), y = g sigmoid(alpha g) (u + 1),
+    output Wd y; a token's expert outputs are summed (f32). gate_up_w [E, 2F, H] (gate rows, then
+    up rows), down_w [E, H, F]."""
+    T, H = x.shape
+    Fd = down_w.shape[2]
+    out = torch.zeros(T, H, dtype=torch.float32, device=x.device)
+    for j in range(topk_ids.shape[1]):
+        for e in topk_ids[:, j].unique().tolist():
+            if e < 0:
+                continue
+            tok = (topk_ids[:, j] == e).nonzero().flatten()
+            h = (x[tok].float() * topk_w[tok, j:j + 1].float()).to(x.dtype).float()
+            gu = h @ gate_up_w[e].float().t()
+            g = gu[:, :Fd].clamp(max=limit)
+            u = gu[:, Fd:].clamp(-limit, limit)
+            y = (g * torch.sigmoid(alpha * g) * (u + 1)).to(x.dtype).float()
+            out[tok] += y @ down_w[e].float().t()
+    return out.to(out_dtype or x.dtype)

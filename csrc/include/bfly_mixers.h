@@ -1,0 +1,77 @@
+// Host-side launch API of the shape-generic kernels: GEMM for any (M, N, K) in bf16 or f32,
+// parallel residual streams (hyper-connections) with offset-weight RMS norms, partial
+// interleaved rotary + paged append, windowed paged attention with kept first tokens and a sink
+// logit, gated linear attention with pooled per-sequence state, score-routed MoE with clamped
+// GLU experts. Every launcher is stream-ordered, allocation-free and synchronisation-free.
+// `f32`: the activation / weight element type is float (else bf16); accumulation, norms,
+// softmax, rotary angles, recurrent state and router scores are f32 in both.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace bfly {
+
+enum AnyAct { ACT_NONE = 0, ACT_RELU2 = 1 };
+
+// out[M, N] = act(x[M, K] w[N, K]^T + bias[N]); `out_f32`: out is float whatever the inputs.
+void launch_gemm_any(const void* x, long ldx, const void* w, long ldw, const void* bias, void* out, long ldo,
+                     int M, int N, int K, int act, bool f32, bool out_f32, hipStream_t s);
+// x <- relu(x)^2 elementwise (n elements)
+void launch_relu2(void* x, long n, bool f32, hipStream_t s);
+
+// xs[t, s, :] = rms(table[ids[t]]) * (w + offset) for every stream s; xs f32 [T, S, W]
+void launch_embed_norm_streams(const int* ids, const void* table, const float* norm_w, float eps, float offset,
+                               float* xs, int T, int S, int W, int vocab, bool f32, hipStream_t s);
+// out[t] = rms(sum_s w_in[s] xs[t, s]) * (w + offset)
+void launch_hc_pre(const float* xs, const float* w_in, const float* norm_w, float eps, float offset, void* out,
+                   int T, int S, int W, bool f32, hipStream_t s);
+// xs[t, r] <- sum_s mix[s, r] xs[t, s] + w_out[r] y[t]   (all streams at once from the old ones)
+void launch_hc_post(float* xs, const void* y, const float* mix, const float* w_out, int T, int S, int W, bool f32,
+                    hipStream_t s);
+// out[i] = rms(sum_s xs[idx[i], s]) * (w + offset); idx == nullptr: every row
+void launch_hc_final(const float* xs, const float* norm_w, float eps, float offset, const long* idx, void* out,
+                     int R, int S, int W, bool f32, hipStream_t s);
+
+// Rotate pairs (2i, 2i+1), i < nrot, of every q and k head by positions[t] * inv_freq[i]; append
+// k / v rows to cache slot slots[t] (>= 0). k == nullptr: q only.
+void launch_rope_partial_kv(void* q, long q_ld, void* k, long k_ld, const void* v, long v_ld, const int* positions,
+                            const float* inv_freq, int nrot, const int* slots, void* k_cache, void* v_cache,
+                            int T, int H, int G, int D, int Dv, int block_size, bool f32, hipStream_t s);
+// row_seq[t] = the sequence whose row range [row_cu[s], row_cu[s+1]) holds row t, else -1
+void launch_row_seq(const int* row_cu, int nseq, int* row_seq, int T, hipStream_t s);
+// Row t of sequence row_seq[t] (-1: padding row, output zero) at position p sees cached keys
+// j <= p with p - j < window or j < keep_first; the softmax denominator includes exp(sink[h]).
+// out [T, H, Dv] contiguous. Dv <= 256.
+void launch_attn_window_paged(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
+                              int max_blocks, const int* row_seq, int nseq, const int* positions, float scale,
+                              int window, int keep_first, const float* sink, void* out, int T, int H, int G, int D,
+                              int Dv, int block_size, bool f32, hipStream_t s);
+
+// Gated linear attention scan over packed rows (see ops.gla_scan). Returns < 0 if D > 256.
+int launch_gla_scan(const void* q, long q_ld, const void* k, long k_ld, const void* v, long v_ld, const void* z,
+                    long z_ld, float* state, const int* state_slots, const int* row_cu, int nseq,
+                    const int* positions, float tau, float q_scale, float* o, int T, int H, int D, int Dv, bool f32,
+                    hipStream_t s);
+// out[t, h * Dv + j] = rms(o[t, h])[j] * w[j] * silu(g[t, h * Dv + j])
+void launch_gla_out(const float* o, const void* g, long g_ld, const float* norm_w, float eps, void* out, int T, int H,
+                    int Dv, bool f32, hipStream_t s);
+
+// Router: f32 logits, scoring 0 softmax / 1 sigmoid, top-k (ties: lowest id), optional renorm.
+// E <= 1024.
+void launch_moe_route_scores(const void* x, long ldx, const void* wr, int top_k, int scoring, bool renorm, int* ids,
+                             float* w, int T, int E, int Hd, bool f32, hipStream_t s);
+// Group the T*K (token, choice) pairs by expert: perm [TK] pair indices grouped by expert,
+// offsets [E + 1], tiles [max_tiles][2] = (expert, first row) of every 64-row tile, ntiles [1].
+void launch_moe_sort(const int* ids, int TK, int E, int* perm, int* offsets, int* tiles, int* ntiles, hipStream_t s);
+int moe_sort_max_tiles(int TK, int E);
+// hmid[r, f] = glu(gate, up) of expert e(r) on (w x) for grouped row r
+void launch_moe_glu_up(const void* x, long ldx, const float* topk_w, int K, const int* perm, const int* offsets,
+                       const int* tiles, const int* ntiles, int max_tiles, const void* gate_up_w, float limit,
+                       float alpha, void* hmid, int Hd, int F, bool f32, hipStream_t s);
+// y[perm[r], :] = down_e(r) hmid[r]     (y f32, pair order)
+void launch_moe_down(const void* hmid, const int* perm, const int* offsets, const int* tiles, const int* ntiles,
+                     int max_tiles, const void* down_w, float* y, int Hd, int F, bool f32, hipStream_t s);
+// out[t] = sum_j y[t * K + j]
+void launch_moe_sum(const float* y, int K, void* out, int T, int Hd, bool f32, hipStream_t s);
+
+}  // namespace bfly

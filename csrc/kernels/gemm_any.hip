@@ -1,0 +1,347 @@
+// Shape-generic GEMM family: any (M, N, K), bf16 or f32 operands, f32 accumulation in K order
+// (the sum of an output element never depends on M or on the other rows of the batch).
+// 64 x 64 output tile, 16-deep K step, 256 threads with a 4 x 4 register block each; operands
+// are staged through LDS as f32 with bounds checks, so no shape or alignment restriction.
+// The same tile core serves the plain projection (bias / squared-ReLU epilogues) and the two
+// grouped expert GEMMs of a score-routed MoE with clamped GLU experts: rows are grouped by
+// expert (moe_sort_kernel), the up kernel gathers token rows scaled by their routing score and
+// applies the GLU to a (gate, up) accumulator pair, the down kernel scatters f32 rows back to
+// (token, choice) order for a fixed-order sum.
+#include <algorithm>
+
+#include "bfly_common.h"
+#include "bfly_mixers.h"
+
+namespace bfly {
+
+namespace {
+
+constexpr int TM = 64, TN = 64, TK = 16, LDP = TM + 4;
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)*p; }
+template <typename T> __device__ __forceinline__ T cvt(float v) { return (T)v; }
+
+// acc[i][j] += sum_k A(row0 + ty*4 + i, k) * B(col0 + tx*4 + j, k); la(r, k) / lb(c, k) return
+// the operand element as float (0 outside the problem).
+template <typename LA, typename LB>
+__device__ __forceinline__ void tile_mac(float (&acc)[4][4], LA la, LB lb, int K, float (*As)[LDP], float (*Bs)[LDP]) {
+  const int tid = threadIdx.x;
+  const int lr = tid >> 2, lk = (tid & 3) * 4;      // staging: row lr, k lk..lk+3
+  const int ty = tid >> 4, tx = tid & 15;
+  for (int k0 = 0; k0 < K; k0 += TK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      As[lk + i][lr] = la(lr, k0 + lk + i);
+      Bs[lk + i][lr] = lb(lr, k0 + lk + i);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < TK; ++kk) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+}
+
+template <typename T, typename TO>
+__global__ __launch_bounds__(256) void gemm_any_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ w,
+                                                       long ldw, const T* __restrict__ bias, TO* __restrict__ out,
+                                                       long ldo, int M, int N, int K, int act) {
+  __shared__ float As[TK][LDP], Bs[TK][LDP];
+  const int row0 = blockIdx.y * TM, col0 = blockIdx.x * TN;
+  float acc[4][4] = {};
+  tile_mac(
+      acc,
+      [&](int r, int k) { return (row0 + r < M && k < K) ? ldf(x + (long)(row0 + r) * ldx + k) : 0.f; },
+      [&](int c, int k) { return (col0 + c < N && k < K) ? ldf(w + (long)(col0 + c) * ldw + k) : 0.f; }, K, As, Bs);
+  const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = row0 + ty * 4 + i;
+    if (r >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = col0 + tx * 4 + j;
+      if (c >= N) continue;
+      float v = acc[i][j];
+      if (bias) v += ldf(bias + c);
+      if (act == ACT_RELU2) { v = fmaxf(v, 0.f); v = v * v; }
+      out[(long)r * ldo + c] = cvt<TO>(v);
+    }
+  }
+}
+
+template <typename T>
+__global__ void relu2_kernel(T* x, long n) {
+  for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    float v = fmaxf((float)x[i], 0.f);
+    x[i] = (T)(v * v);
+  }
+}
+
+// One workgroup. counts -> offsets -> placement (order inside an expert's group is arbitrary:
+// every grouped row is computed on its own and lands at its pair index) -> 64-row tile list.
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int TKp, int E,
+                                                        int* __restrict__ perm, int* __restrict__ offsets,
+                                                        int* __restrict__ tiles, int* __restrict__ ntiles) {
+  __shared__ int cnt[1025], cur[1024];
+  for (int e = threadIdx.x; e <= E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < TKp; i += blockDim.x) {
+    const int e = ids[i];
+    if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0, nt = 0;
+    for (int e = 0; e < E; ++e) {
+      const int c = cnt[e];
+      offsets[e] = run;
+      cur[e] = run;
+      for (int r = 0; r < c; r += 64) {
+        tiles[2 * nt] = e;
+        tiles[2 * nt + 1] = run + r;
+        ++nt;
+      }
+      run += c;
+    }
+    offsets[E] = run;
+    ntiles[0] = nt;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < TKp; i += blockDim.x) {
+    const int e = ids[i];
+    if (e >= 0 && e < E) perm[atomicAdd(&cur[e], 1)] = i;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_glu_up_kernel(const T* __restrict__ x, long ldx,
+                                                         const float* __restrict__ topk_w, int Kc,
+                                                         const int* __restrict__ perm, const int* __restrict__ offsets_e,
+                                                         const int* __restrict__ tiles, const int* __restrict__ ntiles,
+                                                         const T* __restrict__ gu_w, float limit, float alpha,
+                                                         T* __restrict__ hmid, int Hd, int F) {
+  if ((int)blockIdx.y >= ntiles[0]) return;
+  __shared__ float As[TK][LDP], Bs[TK][LDP];
+  __shared__ int tok[TM];
+  __shared__ float wt[TM];
+  const int e = tiles[2 * blockIdx.y], r0 = tiles[2 * blockIdx.y + 1];
+  const int rend = offsets_e[e + 1];
+  const int col0 = blockIdx.x * TN;
+  if (threadIdx.x < TM) {
+    const int r = r0 + threadIdx.x;
+    int p = r < rend ? perm[r] : -1;
+    tok[threadIdx.x] = p < 0 ? -1 : p / Kc;
+    wt[threadIdx.x] = p < 0 ? 0.f : topk_w[p];
+  }
+  __syncthreads();
+  const T* wg = gu_w + (long)e * 2 * F * Hd;
+  const T* wu = wg + (long)F * Hd;
+  // the expert's input is the token row times its routing score, rounded to the activation type
+  auto la = [&](int r, int k) {
+    const int t = tok[r];
+    return (t >= 0 && k < Hd) ? (float)cvt<T>(ldf(x + (long)t * ldx + k) * wt[r]) : 0.f;
+  };
+  float g[4][4] = {}, u[4][4] = {};
+  tile_mac(g, la, [&](int c, int k) { return (col0 + c < F && k < Hd) ? ldf(wg + (long)(col0 + c) * Hd + k) : 0.f; },
+           Hd, As, Bs);
+  tile_mac(u, la, [&](int c, int k) { return (col0 + c < F && k < Hd) ? ldf(wu + (long)(col0 + c) * Hd + k) : 0.f; },
+           Hd, As, Bs);
+  const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r0 + ty * 4 + i;
+    if (r >= rend) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = col0 + tx * 4 + j;
+      if (c >= F) continue;
+      const float gg = fminf(g[i][j], limit);
+      const float uu = fminf(fmaxf(u[i][j], -limit), limit);
+      const float y = gg / (1.f + expf(-alpha * gg)) * (uu + 1.f);
+      hmid[(long)r * F + c] = cvt<T>(y);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ hmid, const int* __restrict__ perm,
+                                                       const int* __restrict__ offsets_e,
+                                                       const int* __restrict__ tiles, const int* __restrict__ ntiles,
+                                                       const T* __restrict__ down_w, float* __restrict__ y, int Hd,
+                                                       int F) {
+  if ((int)blockIdx.y >= ntiles[0]) return;
+  __shared__ float As[TK][LDP], Bs[TK][LDP];
+  const int e = tiles[2 * blockIdx.y], r0 = tiles[2 * blockIdx.y + 1];
+  const int rend = offsets_e[e + 1];
+  const int col0 = blockIdx.x * TN;
+  const T* wd = down_w + (long)e * Hd * F;
+  float acc[4][4] = {};
+  tile_mac(
+      acc, [&](int r, int k) { return (r0 + r < rend && k < F) ? ldf(hmid + (long)(r0 + r) * F + k) : 0.f; },
+      [&](int c, int k) { return (col0 + c < Hd && k < F) ? ldf(wd + (long)(col0 + c) * F + k) : 0.f; }, F, As, Bs);
+  const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r0 + ty * 4 + i;
+    if (r >= rend) continue;
+    const long p = perm[r];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = col0 + tx * 4 + j;
+      if (c < Hd) y[p * Hd + c] = acc[i][j];
+    }
+  }
+}
+
+template <typename T>
+__global__ void moe_sum_kernel(const float* __restrict__ y, int Kc, T* __restrict__ out, long T_, int Hd) {
+  const long n = T_ * Hd;
+  for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const long t = i / Hd;
+    const int c = (int)(i % Hd);
+    float s = 0.f;
+    for (int j = 0; j < Kc; ++j) s += y[(t * Kc + j) * Hd + c];
+    out[i] = (T)s;
+  }
+}
+
+// Router scores of one token per wave: f32 logits (lanes split the hidden dim), softmax or
+// sigmoid, K rounds of arg-max over the experts (ties to the lowest id).
+template <typename T>
+__global__ __launch_bounds__(64) void moe_route_scores_kernel(const T* __restrict__ x, long ldx,
+                                                              const T* __restrict__ wr, int top_k, int scoring,
+                                                              int renorm, int* __restrict__ ids, float* __restrict__ w,
+                                                              int E, int Hd) {
+  __shared__ float sc[1024];
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const T* xr = x + (long)t * ldx;
+  for (int e = 0; e < E; ++e) {
+    float a = 0.f;
+    for (int k = lane; k < Hd; k += 64) a = fmaf(ldf(xr + k), ldf(wr + (long)e * Hd + k), a);
+    a = wave_sum(a);
+    if (lane == 0) sc[e] = a;
+  }
+  __syncthreads();
+  if (scoring == 0) {
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, sc[e]);
+    mx = wave_max(mx);
+    float den = 0.f;
+    for (int e = lane; e < E; e += 64) den += expf(sc[e] - mx);
+    den = wave_sum(den);
+    __syncthreads();
+    for (int e = lane; e < E; e += 64) sc[e] = expf(sc[e] - mx) / den;
+  } else {
+    for (int e = lane; e < E; e += 64) sc[e] = 1.f / (1.f + expf(-sc[e]));
+  }
+  __syncthreads();
+  float sum = 0.f;
+  for (int k = 0; k < top_k; ++k) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float v = sc[e];
+      if (v > bv) { bv = v; bi = e; }      // ascending e: the first maximum wins inside a lane
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    sum += bv;
+    if (lane == 0) {      // (a row of NaN scores selects nothing: id -1)
+      const bool ok = bi < E;
+      ids[(long)t * top_k + k] = ok ? bi : -1;
+      w[(long)t * top_k + k] = ok ? bv : 0.f;
+      if (ok) sc[bi] = -INFINITY;
+    }
+    __syncthreads();
+  }
+  if (renorm && lane == 0)
+    for (int k = 0; k < top_k; ++k) w[(long)t * top_k + k] /= sum;
+}
+
+inline int ew_blocks(long n) { return (int)std::min<long>(4096, std::max<long>(1, (n + 255) / 256)); }
+
+}  // namespace
+
+void launch_gemm_any(const void* x, long ldx, const void* w, long ldw, const void* bias, void* out, long ldo,
+                     int M, int N, int K, int act, bool f32, bool out_f32, hipStream_t s) {
+  if (M <= 0 || N <= 0) return;
+  dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM);
+  if (f32)
+    gemm_any_kernel<float, float><<<grid, 256, 0, s>>>((const float*)x, ldx, (const float*)w, ldw, (const float*)bias,
+                                                       (float*)out, ldo, M, N, K, act);
+  else if (out_f32)
+    gemm_any_kernel<bf16, float><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
+                                                      (float*)out, ldo, M, N, K, act);
+  else
+    gemm_any_kernel<bf16, bf16><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
+                                                     (bf16*)out, ldo, M, N, K, act);
+}
+
+void launch_relu2(void* x, long n, bool f32, hipStream_t s) {
+  if (n <= 0) return;
+  if (f32) relu2_kernel<float><<<ew_blocks(n), 256, 0, s>>>((float*)x, n);
+  else relu2_kernel<bf16><<<ew_blocks(n), 256, 0, s>>>((bf16*)x, n);
+}
+
+void launch_moe_route_scores(const void* x, long ldx, const void* wr, int top_k, int scoring, bool renorm, int* ids,
+                             float* w, int T, int E, int Hd, bool f32, hipStream_t s) {
+  if (T <= 0) return;
+  if (f32)
+    moe_route_scores_kernel<float><<<T, 64, 0, s>>>((const float*)x, ldx, (const float*)wr, top_k, scoring, renorm,
+                                                    ids, w, E, Hd);
+  else
+    moe_route_scores_kernel<bf16><<<T, 64, 0, s>>>((const bf16*)x, ldx, (const bf16*)wr, top_k, scoring, renorm, ids,
+                                                   w, E, Hd);
+}
+
+int moe_sort_max_tiles(int TKp, int E) { return (TKp + 63) / 64 + E; }
+
+void launch_moe_sort(const int* ids, int TKp, int E, int* perm, int* offsets, int* tiles, int* ntiles, hipStream_t s) {
+  moe_sort_kernel<<<1, 1024, 0, s>>>(ids, TKp, E, perm, offsets, tiles, ntiles);
+}
+
+void launch_moe_glu_up(const void* x, long ldx, const float* topk_w, int K, const int* perm, const int* offsets,
+                       const int* tiles, const int* ntiles, int max_tiles, const void* gate_up_w, float limit,
+                       float alpha, void* hmid, int Hd, int F, bool f32, hipStream_t s) {
+  dim3 grid((F + TN - 1) / TN, max_tiles);
+  if (f32)
+    moe_glu_up_kernel<float><<<grid, 256, 0, s>>>((const float*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
+                                                  (const float*)gate_up_w, limit, alpha, (float*)hmid, Hd, F);
+  else
+    moe_glu_up_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
+                                                 (const bf16*)gate_up_w, limit, alpha, (bf16*)hmid, Hd, F);
+}
+
+void launch_moe_down(const void* hmid, const int* perm, const int* offsets, const int* tiles, const int* ntiles,
+                     int max_tiles, const void* down_w, float* y, int Hd, int F, bool f32, hipStream_t s) {
+  dim3 grid((Hd + TN - 1) / TN, max_tiles);
+  if (f32)
+    moe_down_kernel<float><<<grid, 256, 0, s>>>((const float*)hmid, perm, offsets, tiles, ntiles,
+                                                (const float*)down_w, y, Hd, F);
+  else
+    moe_down_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)hmid, perm, offsets, tiles, ntiles, (const bf16*)down_w, y,
+                                               Hd, F);
+}
+
+void launch_moe_sum(const float* y, int K, void* out, int T, int Hd, bool f32, hipStream_t s) {
+  const long n = (long)T * Hd;
+  if (n <= 0) return;
+  if (f32) moe_sum_kernel<float><<<ew_blocks(n), 256, 0, s>>>(y, K, (float*)out, T, Hd);
+  else moe_sum_kernel<bf16><<<ew_blocks(n), 256, 0, s>>>(y, K, (bf16*)out, T, Hd);
+}
+
+}  // namespace bfly

@@ -1,0 +1,311 @@
+// Sequence mixers for heterogeneous layer stacks, generic in head count, head sizes and element
+// type (bf16 or f32 activations / caches; scores, softmax, angles, decays and state are f32):
+//   rope_partial_kv_kernel    interleaved-pair rotary on the first 2 * nrot dims of q / k heads,
+//                             fused with the paged append of k and v (row layouts
+//                             K [blocks, G, BS, D], V [blocks, G, BS, Dv])
+//   attn_window_paged_kernel  attention of packed rows over the paged cache: causal sliding
+//                             window plus the always-visible first `keep_first` positions, and a
+//                             per-head sink logit that only enters the softmax denominator
+//   gla_scan_kernel           gated linear attention S <- diag(a) S + k v^T, o = S^T q with the
+//                             state pooled in per-sequence slots
+//   gla_out_kernel            per-head RMS norm of o, times silu(gate)
+// Rows of a step are packed: sequence s owns rows row_cu[s] .. row_cu[s+1] (one row for a
+// decoded token, several for a prompt chunk), positions[] gives each row's position.
+#include <algorithm>
+
+#include "bfly_common.h"
+#include "bfly_mixers.h"
+
+namespace bfly {
+
+namespace {
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope_partial_kv_kernel(T* __restrict__ q, long q_ld, T* __restrict__ k, long k_ld,
+                                                              const T* __restrict__ v, long v_ld,
+                                                              const int* __restrict__ positions,
+                                                              const float* __restrict__ inv_freq, int nrot,
+                                                              const int* __restrict__ slots, T* __restrict__ k_cache,
+                                                              T* __restrict__ v_cache, int H, int G, int D, int Dv,
+                                                              int bs) {
+  const long t = blockIdx.x;
+  const float p = (float)positions[t];
+  const int slot = (slots && k) ? slots[t] : -1;
+  // rotated pairs of the q heads, then of the k heads
+  const int nq = H * nrot, nk = k ? G * nrot : 0;
+  for (int i = threadIdx.x; i < nq + nk; i += blockDim.x) {
+    const bool isq = i < nq;
+    const int j = isq ? i : i - nq;
+    const int h = j / nrot, r = j % nrot;
+    T* ptr = (isq ? q + t * q_ld : k + t * k_ld) + (long)h * D + 2 * r;
+    const float a = p * inv_freq[r];
+    double sd, cd;
+    sincos((double)a, &sd, &cd);
+    const float c = (float)cd, s = (float)sd;
+    const float u = (float)ptr[0], w = (float)ptr[1];
+    ptr[0] = (T)(u * c - w * s);
+    ptr[1] = (T)(w * c + u * s);
+  }
+  if (slot < 0) return;
+  __syncthreads();      // the rotated k is read back below
+  const long blk = slot / bs, off = slot % bs;
+  for (int i = threadIdx.x; i < G * D; i += blockDim.x) {
+    const int g = i / D, d = i % D;
+    k_cache[((blk * G + g) * bs + off) * D + d] = k[t * k_ld + i];
+  }
+  for (int i = threadIdx.x; i < G * Dv; i += blockDim.x) {
+    const int g = i / Dv, d = i % Dv;
+    v_cache[((blk * G + g) * bs + off) * Dv + d] = v[t * v_ld + i];
+  }
+}
+
+// One wave per (row, query head). Keys are visited 64 at a time (one per lane) with an online
+// softmax seeded by the sink: m = sink, l = 1, acc = 0, so the sink counts once in the
+// denominator and has no value. Lane `l` then owns output dims l, l + 64, ... (Dv <= 256).
+constexpr int kMaxDvLane = 4;
+
+template <typename T>
+__global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restrict__ q, long q_ld,
+                                                               const T* __restrict__ k_cache,
+                                                               const T* __restrict__ v_cache,
+                                                               const int* __restrict__ tables, int max_blocks,
+                                                               const int* __restrict__ row_seq,
+                                                               const int* __restrict__ positions, float scale,
+                                                               int window, int keep_first,
+                                                               const float* __restrict__ sink, T* __restrict__ out,
+                                                               int H, int G, int D, int Dv, int bs) {
+  extern __shared__ float smem[];      // q [D] | p [64] | key row base index [64] (as int)
+  float* sq = smem;
+  float* sp = smem + D;
+  long* sj = reinterpret_cast<long*>(smem + D + 64 + ((D & 1) ? 1 : 0));
+  const long t = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const int g = h / (H / G);
+  const int s = row_seq[t];
+  if (s < 0) {       // padding row of a fixed-shape step
+    for (int d = lane; d < Dv; d += 64) out[(t * H + h) * Dv + d] = (T)0.f;
+    return;
+  }
+  const int p = positions[t];
+  const int* tab = tables + (long)s * max_blocks;
+  for (int d = lane; d < D; d += 64) sq[d] = (float)q[t * q_ld + (long)h * D + d];
+  __syncthreads();
+  const int lo = max(0, p - window + 1);
+  const int n1 = min(keep_first, lo);          // kept first positions outside the window
+  const int total = n1 + (p - lo + 1);
+  float m = sink[h], l = 1.f;
+  float acc[kMaxDvLane] = {0.f, 0.f, 0.f, 0.f};
+  for (int i0 = 0; i0 < total; i0 += 64) {
+    const int i = i0 + lane;
+    float sc = -INFINITY;
+    long kv_row = 0;
+    if (i < total) {
+      const int j = i < n1 ? i : lo + (i - n1);
+      kv_row = ((long)tab[j / bs] * G + g) * bs + (j % bs);
+      const T* kr = k_cache + kv_row * D;
+      float a = 0.f;
+      for (int d = 0; d < D; ++d) a = fmaf(sq[d], (float)kr[d], a);
+      sc = a * scale;
+    }
+    const float mn = fmaxf(m, wave_max(sc));
+    const float pe = i < total ? expf(sc - mn) : 0.f;
+    const float corr = expf(m - mn);
+    l = l * corr + wave_sum(pe);
+    m = mn;
+    __syncthreads();
+    sp[lane] = pe;
+    sj[lane] = kv_row;
+    __syncthreads();
+    const int cnt = min(64, total - i0);
+#pragma unroll
+    for (int c = 0; c < kMaxDvLane; ++c) {
+      const int d = lane + 64 * c;
+      if (d >= Dv) break;
+      float a = acc[c] * corr;
+      for (int x = 0; x < cnt; ++x) a = fmaf(sp[x], (float)v_cache[sj[x] * Dv + d], a);
+      acc[c] = a;
+    }
+  }
+  const float inv = 1.f / l;
+#pragma unroll
+  for (int c = 0; c < kMaxDvLane; ++c) {
+    const int d = lane + 64 * c;
+    if (d < Dv) out[(t * H + h) * Dv + d] = (T)(acc[c] * inv);
+  }
+}
+
+// row -> sequence map of a packed step (rows outside every sequence: -1)
+__global__ void row_seq_kernel(const int* __restrict__ row_cu, int nseq, int* __restrict__ row_seq, int T) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  int s = -1;
+  for (int i = 0; i < nseq; ++i)
+    if (t >= row_cu[i] && t < row_cu[i + 1]) { s = i; break; }
+  row_seq[t] = s;
+}
+
+// Workgroup = (sequence, head, 64-column slice of Dv), 4 waves. Wave w keeps rows d = w, w+4, ...
+// of the slice's state in registers (NR per lane, lane = column); per token the decays, keys and
+// queries of the head are staged in LDS, each wave updates its rows and the four partial
+// outputs are summed through LDS.
+template <typename T, int NR>
+__global__ __launch_bounds__(256) void gla_scan_kernel(const T* __restrict__ q, long q_ld, const T* __restrict__ k,
+                                                       long k_ld, const T* __restrict__ v, long v_ld,
+                                                       const T* __restrict__ z, long z_ld, float* __restrict__ state,
+                                                       const int* __restrict__ state_slots,
+                                                       const int* __restrict__ row_cu,
+                                                       const int* __restrict__ positions, float inv_tau,
+                                                       float q_scale, float* __restrict__ o, int H, int D, int Dv) {
+  __shared__ float sa[256], sk[256], sq[256], part[4][64];
+  const int s = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * 64;
+  const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int col = c0 + lane;
+  const bool live = col < Dv;
+  const int r0 = row_cu[s], r1 = row_cu[s + 1];
+  const int slot = state_slots[s];
+  if (r1 <= r0) return;
+  if (slot < 0) {      // padding sequence of a fixed-shape step: defined output, no state
+    if (w == 0 && live)
+      for (int t = r0; t < r1; ++t) o[((long)t * H + h) * Dv + col] = 0.f;
+    return;
+  }
+  float* S = state + ((long)slot * H + h) * D * Dv;
+  float st[NR];
+  const bool fresh = positions[r0] == 0;
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    const int d = w + 4 * i;
+    st[i] = (!fresh && live && d < D) ? S[(long)d * Dv + col] : 0.f;
+  }
+  for (int t = r0; t < r1; ++t) {
+    if ((int)threadIdx.x < D) {
+      const int d = threadIdx.x;
+      const float zz = (float)z[(long)t * z_ld + (long)h * D + d];
+      // log sigmoid(z) = -softplus(-z), stable on both sides
+      const float ls = zz < 0.f ? zz - log1pf(expf(zz)) : -log1pf(expf(-zz));
+      sa[d] = expf(ls * inv_tau);
+      sk[d] = (float)k[(long)t * k_ld + (long)h * D + d];
+      sq[d] = (float)q[(long)t * q_ld + (long)h * D + d] * q_scale;
+    }
+    const float vv = live ? (float)v[(long)t * v_ld + (long)h * Dv + col] : 0.f;
+    __syncthreads();
+    float po = 0.f;
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const int d = w + 4 * i;
+      if (d < D) {
+        st[i] = fmaf(sa[d], st[i], sk[d] * vv);
+        po = fmaf(sq[d], st[i], po);
+      }
+    }
+    part[w][lane] = po;
+    __syncthreads();
+    if (w == 0 && live) o[((long)t * H + h) * Dv + col] = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const int d = w + 4 * i;
+      if (d < D) S[(long)d * Dv + col] = st[i];
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(64) void gla_out_kernel(const float* __restrict__ o, const T* __restrict__ g, long g_ld,
+                                                     const float* __restrict__ norm_w, float eps, T* __restrict__ out,
+                                                     int H, int Dv) {
+  const long t = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const float* row = o + (t * H + h) * Dv;
+  float ss = 0.f;
+  for (int d = lane; d < Dv; d += 64) ss = fmaf(row[d], row[d], ss);
+  ss = wave_sum(ss);
+  const float r = 1.f / sqrtf(ss / (float)Dv + eps);
+  for (int d = lane; d < Dv; d += 64) {
+    const float gg = (float)g[t * g_ld + (long)h * Dv + d];
+    const float y = row[d] * r * norm_w[d];
+    out[(t * H + h) * Dv + d] = (T)(y * (gg / (1.f + expf(-gg))));
+  }
+}
+
+}  // namespace
+
+void launch_rope_partial_kv(void* q, long q_ld, void* k, long k_ld, const void* v, long v_ld, const int* positions,
+                            const float* inv_freq, int nrot, const int* slots, void* k_cache, void* v_cache,
+                            int T, int H, int G, int D, int Dv, int block_size, bool f32, hipStream_t s) {
+  if (T <= 0) return;
+  if (f32)
+    rope_partial_kv_kernel<float><<<T, 256, 0, s>>>((float*)q, q_ld, (float*)k, k_ld, (const float*)v, v_ld, positions,
+                                                    inv_freq, nrot, slots, (float*)k_cache, (float*)v_cache, H, G, D,
+                                                    Dv, block_size);
+  else
+    rope_partial_kv_kernel<bf16><<<T, 256, 0, s>>>((bf16*)q, q_ld, (bf16*)k, k_ld, (const bf16*)v, v_ld, positions,
+                                                   inv_freq, nrot, slots, (bf16*)k_cache, (bf16*)v_cache, H, G, D, Dv,
+                                                   block_size);
+}
+
+void launch_row_seq(const int* row_cu, int nseq, int* row_seq, int T, hipStream_t s) {
+  if (T <= 0) return;
+  row_seq_kernel<<<(T + 255) / 256, 256, 0, s>>>(row_cu, nseq, row_seq, T);
+}
+
+void launch_attn_window_paged(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
+                              int max_blocks, const int* row_seq, int nseq, const int* positions, float scale,
+                              int window, int keep_first, const float* sink, void* out, int T, int H, int G, int D,
+                              int Dv, int block_size, bool f32, hipStream_t s) {
+  if (T <= 0) return;
+  (void)nseq;
+  dim3 grid(T, H);
+  const size_t sm = (size_t)(D + 64 + 2) * sizeof(float) + 64 * sizeof(long);
+  if (f32)
+    attn_window_paged_kernel<float><<<grid, 64, sm, s>>>((const float*)q, q_ld, (const float*)k_cache,
+                                                         (const float*)v_cache, tables, max_blocks, row_seq, positions,
+                                                         scale, window, keep_first, sink, (float*)out, H, G, D, Dv,
+                                                         block_size);
+  else
+    attn_window_paged_kernel<bf16><<<grid, 64, sm, s>>>((const bf16*)q, q_ld, (const bf16*)k_cache,
+                                                        (const bf16*)v_cache, tables, max_blocks, row_seq, positions,
+                                                        scale, window, keep_first, sink, (bf16*)out, H, G, D, Dv,
+                                                        block_size);
+}
+
+template <typename T>
+static int gla_scan_t(const T* q, long q_ld, const T* k, long k_ld, const T* v, long v_ld, const T* z, long z_ld,
+                      float* state, const int* state_slots, const int* row_cu, int nseq, const int* positions,
+                      float tau, float q_scale, float* o, int H, int D, int Dv, hipStream_t s) {
+  dim3 grid(nseq, H, (Dv + 63) / 64);
+  const float it = 1.f / tau;
+#define BFLY_GLA(NR)                                                                                              \
+  gla_scan_kernel<T, NR><<<grid, 256, 0, s>>>(q, q_ld, k, k_ld, v, v_ld, z, z_ld, state, state_slots, row_cu, positions, \
+                                              it, q_scale, o, H, D, Dv)
+  if (D <= 32) BFLY_GLA(8);
+  else if (D <= 64) BFLY_GLA(16);
+  else if (D <= 128) BFLY_GLA(32);
+  else if (D <= 256) BFLY_GLA(64);
+  else return -1;
+#undef BFLY_GLA
+  return 0;
+}
+
+int launch_gla_scan(const void* q, long q_ld, const void* k, long k_ld, const void* v, long v_ld, const void* z,
+                    long z_ld, float* state, const int* state_slots, const int* row_cu, int nseq,
+                    const int* positions, float tau, float q_scale, float* o, int T, int H, int D, int Dv, bool f32,
+                    hipStream_t s) {
+  if (T <= 0 || nseq <= 0) return 0;
+  if (f32)
+    return gla_scan_t<float>((const float*)q, q_ld, (const float*)k, k_ld, (const float*)v, v_ld, (const float*)z, z_ld,
+                             state, state_slots, row_cu, nseq, positions, tau, q_scale, o, H, D, Dv, s);
+  return gla_scan_t<bf16>((const bf16*)q, q_ld, (const bf16*)k, k_ld, (const bf16*)v, v_ld, (const bf16*)z, z_ld, state,
+                          state_slots, row_cu, nseq, positions, tau, q_scale, o, H, D, Dv, s);
+}
+
+void launch_gla_out(const float* o, const void* g, long g_ld, const float* norm_w, float eps, void* out, int T, int H,
+                    int Dv, bool f32, hipStream_t s) {
+  if (T <= 0) return;
+  dim3 grid(T, H);
+  if (f32) gla_out_kernel<float><<<grid, 64, 0, s>>>(o, (const float*)g, g_ld, norm_w, eps, (float*)out, H, Dv);
+  else gla_out_kernel<bf16><<<grid, 64, 0, s>>>(o, (const bf16*)g, g_ld, norm_w, eps, (bf16*)out, H, Dv);
+}
+
+}  // namespace bfly

@@ -17,7 +17,11 @@ namespace bfly_rt {
 
 void register_kv_manager(py::module_& m) {
   py::class_<KVBlockManager>(m, "KVBlockManager")
-      .def(py::init<int, int>(), py::arg("num_blocks"), py::arg("block_size"))
+      .def(py::init<int, int, int>(), py::arg("num_blocks"), py::arg("block_size"), py::arg("state_slots") = 0)
+      .def_property_readonly("num_state_slots", &KVBlockManager::num_state_slots)
+      .def_property_readonly("num_free_state_slots", &KVBlockManager::num_free_state_slots)
+      .def("state_slot", &KVBlockManager::state_slot)
+      .def("state_slots_of", &KVBlockManager::state_slots_of)
       .def_property_readonly("num_blocks", &KVBlockManager::num_blocks)
       .def_property_readonly("block_size", &KVBlockManager::block_size)
       .def_property_readonly("num_free", &KVBlockManager::num_free)

@@ -39,12 +39,31 @@ inline uint64_t kv_block_hash(uint64_t prev, const int32_t* tok, int n) {
 
 class KVBlockManager {
  public:
-  KVBlockManager(int num_blocks, int block_size)
+  // `state_slots` > 0: every live sequence also owns one slot of a fixed pool of per-sequence
+  // recurrent-state rows (models with linear-attention / recurrent layers keep their running
+  // state there). A slot is taken when the sequence is registered and returned by free(); the
+  // kernels treat a sequence whose step starts at position 0 as having zero state, so a slot
+  // needs no clearing between owners.
+  KVBlockManager(int num_blocks, int block_size, int state_slots = 0)
       : num_blocks_(num_blocks), block_size_(block_size), refcnt_(num_blocks, 0),
-        hash_(num_blocks, 0), lru_pos_(num_blocks) {
-    if (num_blocks <= 0 || block_size <= 0) throw std::invalid_argument("bad KV geometry");
+        hash_(num_blocks, 0), lru_pos_(num_blocks), state_slots_(state_slots) {
+    if (num_blocks <= 0 || block_size <= 0 || state_slots < 0) throw std::invalid_argument("bad KV geometry");
     free_.reserve(num_blocks);
     for (int b = num_blocks - 1; b >= 0; --b) free_.push_back(b);
+    for (int s = state_slots - 1; s >= 0; --s) free_states_.push_back(s);
+  }
+
+  int num_state_slots() const { return state_slots_; }
+  int num_free_state_slots() const { return (int)free_states_.size(); }
+  // A new sequence can be registered (state pool off, or a slot is free).
+  bool state_available() const { return state_slots_ == 0 || !free_states_.empty(); }
+  // The sequence's recurrent-state slot (-1: the pool is off).
+  int32_t state_slot(int64_t sid) const { return cget(sid).state; }
+  std::vector<int32_t> state_slots_of(const std::vector<int64_t>& sids) const {
+    std::vector<int32_t> out;
+    out.reserve(sids.size());
+    for (int64_t sid : sids) out.push_back(cget(sid).state);
+    return out;
   }
 
   int num_blocks() const { return num_blocks_; }
@@ -73,7 +92,10 @@ class KVBlockManager {
   std::vector<int32_t> allocate_prefixed(int64_t sid, const std::vector<uint64_t>& hashes, int nblocks,
                                          int64_t tokens) {
     if (seqs_.count(sid)) throw std::invalid_argument("sequence already allocated");
+    if (nblocks > 0 && state_slots_ > 0)
+      throw std::invalid_argument("cached prefix pages cannot restore a recurrent state");
     Seq s;
+    s.state = take_state();
     for (int i = 0; i < nblocks; ++i) {
       const int b = cached_.at(hashes[i]);
       if (refcnt_[b] == 0) lru_.erase(lru_pos_[b]);   // parked page comes back to life
@@ -99,7 +121,7 @@ class KVBlockManager {
   bool has(int64_t sid) const { return seqs_.count(sid) != 0; }
 
   int blocks_needed(int64_t tokens) const { return (int)((tokens + block_size_ - 1) / block_size_); }
-  bool can_allocate(int64_t tokens) const { return blocks_needed(tokens) <= num_free(); }
+  bool can_allocate(int64_t tokens) const { return blocks_needed(tokens) <= num_free() && state_available(); }
 
   // Register a sequence with `tokens` tokens to cache; returns their slots.
   std::vector<int32_t> allocate(int64_t sid, int64_t tokens) {
@@ -107,6 +129,7 @@ class KVBlockManager {
     const int nb = blocks_needed(tokens);
     if (nb > num_free()) throw std::runtime_error("KV cache out of blocks");
     Seq s;
+    s.state = take_state();
     s.blocks.reserve(nb + 4);
     for (int i = 0; i < nb; ++i) s.blocks.push_back(take());
     s.len = tokens;
@@ -167,6 +190,7 @@ class KVBlockManager {
   void fork(int64_t parent, int64_t child) {
     const Seq& p = cget(parent);
     if (seqs_.count(child)) throw std::invalid_argument("child exists");
+    if (state_slots_ > 0) throw std::invalid_argument("fork: a recurrent state cannot be shared");
     Seq c = p;
     for (int b : c.blocks) ++refcnt_[b];
     seqs_.emplace(child, std::move(c));
@@ -176,6 +200,7 @@ class KVBlockManager {
     auto it = seqs_.find(sid);
     if (it == seqs_.end()) return;
     for (int b : it->second.blocks) release(b);
+    if (it->second.state >= 0) free_states_.push_back(it->second.state);
     seqs_.erase(it);
   }
 
@@ -212,7 +237,15 @@ class KVBlockManager {
   struct Seq {
     std::vector<int> blocks;
     int64_t len = 0;
+    int32_t state = -1;   // recurrent-state slot
   };
+  int32_t take_state() {
+    if (state_slots_ == 0) return -1;
+    if (free_states_.empty()) throw std::runtime_error("out of recurrent-state slots");
+    const int32_t s = free_states_.back();
+    free_states_.pop_back();
+    return s;
+  }
   int take() {
     int b;
     if (!free_.empty()) {
@@ -258,6 +291,8 @@ class KVBlockManager {
   std::vector<std::list<int>::iterator> lru_pos_;
   std::unordered_map<uint64_t, int> cached_;          // hash -> page
   std::unordered_map<int64_t, Seq> seqs_;
+  int state_slots_;
+  std::vector<int32_t> free_states_;                  // LIFO: a freed slot is the next one taken
 };
 
 }  // namespace bfly_rt

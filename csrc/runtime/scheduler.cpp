@@ -34,6 +34,7 @@ void register_scheduler(py::module_& m) {
       .def("on_token", &Scheduler::on_token)
       .def("finish", &Scheduler::finish)
       .def("schedule", &Scheduler::schedule)
+      .def("schedule_script", &Scheduler::schedule_script, py::arg("entries"))
       .def_property_readonly("num_waiting", &Scheduler::num_waiting)
       .def_property_readonly("num_running", &Scheduler::num_running)
       .def("running", &Scheduler::running)

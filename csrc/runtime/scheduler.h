@@ -76,7 +76,8 @@ class Scheduler {
     return kv_.allocate(sid, prompt_len);
   }
   bool can_admit_prefilled(int64_t prompt_len) const {
-    return (int)running_.size() < max_batch_ && kv_.blocks_needed(prompt_len + 1) <= kv_.num_free();
+    return (int)running_.size() < max_batch_ && kv_.blocks_needed(prompt_len + 1) <= kv_.num_free() &&
+           kv_.state_available();
   }
 
 
@@ -97,6 +98,59 @@ class Scheduler {
   std::vector<int64_t> running() const { return running_; }
   std::vector<int64_t> waiting() const { return std::vector<int64_t>(waiting_.begin(), waiting_.end()); }
 
+  // Replay of a recorded schedule: the caller names, per step, the sequences that run and how
+  // many of their next tokens each brings (a trace of a serving run, a test of cache and state
+  // handling under a fixed interleaving). No admission policy and no preemption: a sequence is
+  // registered at its first entry (pages, and a recurrent-state slot if the manager pools them),
+  // stays running while steps leave it out, and is released by finish(). One token of a sequence
+  // that already holds tokens is a decode row; everything else is a prompt chunk that attends to
+  // what the sequence has cached. The plan has the mixed-step layout (decode rows first).
+  StepPlan schedule_script(const std::vector<std::pair<int64_t, int64_t>>& entries) {
+    StepPlan plan;
+    int fresh_pages = 0, fresh_states = 0;
+    for (const auto& [sid, n] : entries) {
+      if (n <= 0) throw std::invalid_argument("scripted entry without tokens");
+      if (kv_.has(sid)) {
+        fresh_pages += kv_.extend_blocks(sid, n);
+      } else {
+        fresh_pages += kv_.blocks_needed(n);
+        ++fresh_states;
+      }
+    }
+    if (fresh_pages > kv_.num_free()) throw std::runtime_error("scripted step does not fit the KV cache");
+    if (kv_.num_state_slots() > 0 && fresh_states > kv_.num_free_state_slots())
+      throw std::runtime_error("scripted step needs more recurrent-state slots than are free");
+    if ((int)running_.size() + fresh_states > max_batch_) throw std::runtime_error("scripted step exceeds max_batch");
+    for (const auto& [sid, n] : entries) {      // decode rows
+      if (n != 1 || !kv_.has(sid) || kv_.length(sid) == 0) continue;
+      plan.decode_positions.push_back((int32_t)kv_.length(sid));
+      auto [slot, src, dst] = kv_.append_slot(sid);
+      plan.seq_ids.push_back(sid);
+      plan.decode_slots.push_back(slot);
+      if (src >= 0) plan.cow.emplace_back(src, dst);
+    }
+    plan.num_decode = (int)plan.seq_ids.size();
+    for (const auto& [sid, n] : entries) {      // prompt chunks
+      const bool known = kv_.has(sid);
+      if (known && std::find(plan.seq_ids.begin(), plan.seq_ids.begin() + plan.num_decode, sid) !=
+                       plan.seq_ids.begin() + plan.num_decode)
+        continue;
+      const int64_t start = known ? kv_.length(sid) : 0;
+      if (!known) {
+        info_[sid] = Info{0, 0, 0, true, {}};
+        running_.push_back(sid);
+      }
+      plan.seq_ids.push_back(sid);
+      plan.prefill_starts.push_back(start);
+      plan.prefill_lens.push_back(n);
+      plan.prefill_slots.push_back(known ? kv_.extend(sid, n) : kv_.allocate(sid, n));
+      plan.prefill_final.push_back(true);
+    }
+    const bool has_prefill = (int)plan.seq_ids.size() > plan.num_decode;
+    plan.kind = plan.num_decode > 0 ? (has_prefill ? 3 : 2) : (has_prefill ? 1 : 0);
+    return plan;
+  }
+
   StepPlan schedule() {
     if (mixed_) return schedule_mixed();
     StepPlan plan;
@@ -109,7 +163,7 @@ class Scheduler {
       const int64_t len = in.prompt_len + in.generated;   // recompute after preemption
       if (len > budget && !plan.seq_ids.empty()) break;
       const int need = kv_.blocks_needed(len + 1);
-      if (need > free_pages) break;
+      if (need > free_pages || !kv_.state_available()) break;
       waiting_.pop_front();
       plan.seq_ids.push_back(sid);
       plan.prefill_lens.push_back(len);
@@ -213,7 +267,7 @@ class Scheduler {
       const bool fin = start + n == target;
       // fresh pages for the chunk (+ one decode page when it completes the prompt); the
       // matched pages may be parked ones, which also count as free: reserve them too
-      if (kv_.blocks_needed(start + n + (fin ? 1 : 0)) > kv_.num_free()) break;
+      if (kv_.blocks_needed(start + n + (fin ? 1 : 0)) > kv_.num_free() || !kv_.state_available()) break;
       waiting_.pop_front();
       running_.push_back(sid);
       plan.seq_ids.push_back(sid);
