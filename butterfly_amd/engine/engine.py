@@ -998,16 +998,15 @@ class LLMEngine:
         single-stage engines only (EngineConfig.async_decode = False)."""
         if self.async_pp or self.mesh.world_size != 1:
             raise RuntimeError("replay_step needs a synchronous single-rank engine (async_decode=False)")
-        sched = []
-        for rid, toks, _ in entries:
-            req = self.requests.get(rid)
-            if req is None:
-                req = self.requests[rid] = Request(rid, [], SamplingParams(max_tokens=1), arrival=time.perf_counter())
-            req.prompt.extend(int(t) for t in toks)
-            sched.append((rid, len(toks)))
+        sched = [(rid, len(toks)) for rid, toks, _ in entries]
         logits = None
         if sched:
-            plan = self.scheduler.schedule_script(sched)
+            plan = self.scheduler.schedule_script(sched)     # raises before it changes anything
+            for rid, toks, _ in entries:
+                req = self.requests.get(rid)
+                if req is None:
+                    req = self.requests[rid] = Request(rid, [], SamplingParams(max_tokens=1), arrival=time.perf_counter())
+                req.prompt.extend(int(t) for t in toks)
             if plan.cow:
                 self.kv.copy_blocks(list(plan.cow))
             rows = self._plan_rows(plan)

@@ -411,6 +411,16 @@ def sample(logits, temps=None, seeds=None, vstart: int = 0, out_ids=None, out_sc
         out_ids = _empty(rows, dtype=torch.int32, device=logits.device)
     if out_scores is None:
         out_scores = _empty(rows, dtype=torch.float32, device=logits.device)
+    if logits.dtype == torch.float32:
+        # f32 serving mode: greedy rows pick from the f32 values themselves; stochastic rows go
+        # through the bf16 sampler on a rounded copy (16-byte rows)
+        if temps is None and thresh is None:
+            torch.ops.bfly.sample_greedy_f32(logits, vstart, out_ids, out_scores, check_finite)
+            return out_ids, out_scores
+        n = logits.shape[1]
+        buf = torch.empty(rows, (n + 7) // 8 * 8, dtype=torch.bfloat16, device=logits.device)
+        buf[:, :n].copy_(logits)
+        logits = buf[:, :n]
     ws = _arena.get(logits.device, "sample", rows * 64, torch.int64)
     torch.ops.bfly.sample(logits, temps, seeds, vstart, out_ids, out_scores, ws, thresh, check_finite)
     return out_ids, out_scores

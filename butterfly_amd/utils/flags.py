@@ -63,6 +63,8 @@ define("BFLY_ATTN_XCD", 1, int, "prefill attention: XCD-aware item walk (0: plai
 define("BFLY_ATTN_TRACE", "", str, "set: the prefill attention kernel stamps its item phases into the LSE buffer "
        "instead of writing results (tools/attn_trace.py; read by the kernel library)")
 define("BFLY_KERNEL_LIB", "", str, "path of another build of the kernel library (same-box A/B runs of kernel changes)")
+define("BFLY_TRACE_DEVICE", "", str, "device of `trace-run` (default: the GPU, which it requires; \"cpu\" replays a "
+       "schedule through the reference ops)")
 define("BFLY_LOG_JSON", False, _bool, "emit log records as one JSON object per line")
 define("BFLY_RESTART", 0, int, "restart attempt of this job (set by `launch --max-restarts`; 0 = first run)")
 define("BFLY_ATTN_PAGED_LDS", True, _bool, "paged-prefix prefill attention: the LDS-staged kernel for chunks of "

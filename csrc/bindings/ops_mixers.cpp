@@ -6,6 +6,7 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/library.h>
 
+#include "bfly_kernels.h"
 #include "bfly_mixers.h"
 
 namespace {
@@ -77,7 +78,7 @@ void hc_post(Tensor& xs, const Tensor& y, const Tensor& mix, const Tensor& w_out
   CHK_GPU(xs); CHK_F32(xs); CHK_F32(mix); CHK_F32(w_out);
   TORCH_CHECK(xs.dim() == 3 && y.dim() == 2 && y.is_contiguous(), "hc_post: layouts");
   const int64_t T = xs.size(0), S = xs.size(1), W = xs.size(2);
-  TORCH_CHECK(S <= 8, "hc_post: at most 8 residual streams");
+  TORCH_CHECK(S <= 16, "hc_post: at most 16 residual streams");
   TORCH_CHECK(mix.numel() == S * S && w_out.numel() == S && y.size(0) == T && y.size(1) == W, "hc_post: shapes");
   bfly::launch_hc_post(xs.data_ptr<float>(), y.data_ptr(), mix.data_ptr<float>(), w_out.data_ptr<float>(), (int)T,
                        (int)S, (int)W, is_f32(y), cur_stream());
@@ -241,9 +242,19 @@ void moe_glu_ffn(const Tensor& x, const Tensor& topk_ids, const Tensor& topk_w, 
   bfly::launch_moe_sum(y.data_ptr<float>(), (int)K, out.data_ptr(), (int)T, (int)Hd, f32, s);
 }
 
+void sample_greedy_f32(const Tensor& logits, int64_t vstart, Tensor& out_ids, Tensor& out_scores, bool check_finite) {
+  CHK_GPU(logits); CHK_I32(out_ids); CHK_F32(out_scores);
+  TORCH_CHECK(logits.scalar_type() == at::kFloat && logits.dim() == 2 && logits.stride(1) == 1, "sample_greedy_f32: logits");
+  const int64_t rows = logits.size(0);
+  TORCH_CHECK(out_ids.numel() == rows && out_scores.numel() == rows && logits.size(1) >= 1, "sample_greedy_f32: outputs");
+  bfly::launch_sample_greedy_f32(logits.data_ptr<float>(), logits.stride(0), (int)rows, (int)logits.size(1), (int)vstart,
+                                 out_ids.data_ptr<int>(), out_scores.data_ptr<float>(), cur_stream(), check_finite ? 1 : 0);
+}
+
 }  // namespace
 
 TORCH_LIBRARY_FRAGMENT(bfly, m) {
+  m.def("sample_greedy_f32(Tensor logits, int vstart, Tensor(a!) out_ids, Tensor(b!) out_scores, bool check_finite) -> ()");
   m.def("gemm_any(Tensor x, Tensor w, Tensor? bias, int act, Tensor(a!) out) -> ()");
   m.def("relu2_(Tensor(a!) x) -> ()");
   m.def("embed_norm_streams(Tensor ids, Tensor table, Tensor norm_w, float eps, float offset, Tensor(a!) xs) -> ()");
@@ -265,6 +276,7 @@ TORCH_LIBRARY_FRAGMENT(bfly, m) {
 }
 
 TORCH_LIBRARY_IMPL(bfly, CUDA, m) {
+  m.impl("sample_greedy_f32", &sample_greedy_f32);
   m.impl("gemm_any", &gemm_any);
   m.impl("relu2_", &relu2_);
   m.impl("embed_norm_streams", &embed_norm_streams);

@@ -91,6 +91,8 @@ void launch_sample(const bf16* logits, long row_stride, int rows, int V, int vst
                    float* out_scores, hipStream_t stream, const float* thresh = nullptr,
                    int check_finite = 0);
 // TP merge of per-shard winners: pair [rows][2] f32 (score, id); allp [tp][rows][2] -> ids
+void launch_sample_greedy_f32(const float* logits, long row_stride, int rows, int V, int vstart, int* out_ids,
+                              float* out_scores, hipStream_t stream, int check_finite);
 void launch_sample_pack(const float* scores, const int* ids, float* pair, int rows, hipStream_t stream);
 void launch_sample_merge(const float* allp, int tp, int rows, int* out, hipStream_t stream);
 // exact top-k / top-p thresholds by radix select (sample.hip): state [rows, 8] f32 bits,

@@ -11,7 +11,7 @@ namespace bfly {
 
 namespace {
 
-constexpr int kMaxStreams = 8;
+constexpr int kMaxStreams = 16;
 
 template <typename T>
 __global__ __launch_bounds__(256) void embed_norm_streams_kernel(const int* __restrict__ ids, const T* __restrict__ table,
