@@ -96,7 +96,21 @@ same = sum(int(a == b) for a, b in zip(out_free, single))
 # bf16 partial sums in a different order can flip a near-tie late in a free-running sequence,
 # so the hard checks are teacher-forced: EVERY step's (prefill and each decode step) logits
 # within bf16 tolerance of the single GPU's, plus identical first tokens and prefill logits
-first_ok = all(a[0] == b[0] for a, b in zip(out_free, single))
+# (a first token may differ only where the single-GPU logits of the two candidates are a near-tie:
+# closer than the per-step logit tolerance allows a sharded run to resolve)
+def _first_same(i, a, b):
+    if a[0] == b[0]:
+        return True
+    ref = ref_logits.get((i, 0))
+    if ref is None:
+        return False
+    gap = float(ref[b[0]] - ref[a[0]])
+    print(f"rank {rank} first token of prompt {i}: sharded {a[0]} vs single {b[0]}, single-GPU logit gap {gap:.3e} "
+          f"(logit rms {float(ref.norm() / ref.numel() ** 0.5):.3e})", flush=True)
+    return 0.0 <= gap < 3e-2 * float(ref.norm() / ref.numel() ** 0.5)
+
+
+first_ok = all(_first_same(i, a, b) for i, (a, b) in enumerate(zip(out_free, single)))
 samplers = eng.model.last
 steps_ok = (not samplers) or (len(step_err) == params.max_tokens and max(step_err.values()) < 3e-2)
 ok = first_ok and rel < 2e-2 and steps_ok
