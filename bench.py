@@ -92,6 +92,11 @@ def build_parser() -> argparse.ArgumentParser:
                     help="single-stage layouts: host waits for each step's tokens before scheduling the "
                          "next (default: EngineConfig.async_decode, the next step overlaps the host work)")
     ap.add_argument("--out", default=None, help="also write the JSON line here")
+    ap.add_argument("--mixer-compare", default=None, metavar="SIZES",
+                    help="instead of the headline run: prefill and decode throughput of a Nesizen stack "
+                         "(windowed attention, shared keys, gated linear attention, sigmoid MoE) beside a "
+                         "Mixtral stack of equal width, depth, heads and experts, random weights, one GPU; "
+                         "SIZES = comma list of s, m, l (width 1024 / 2048 / 4096)")
     return ap
 
 
@@ -128,9 +133,101 @@ def main(argv=None) -> int:
     argv = list(sys.argv[1:] if argv is None else argv)
     a = build_parser().parse_args(argv)
     resolve(a)
+    if a.mixer_compare:
+        return run_mixer_compare(a)
     if a.gpus > 1 and "WORLD_SIZE" not in os.environ:
         return self_launch(a, argv)
     return run(a)
+
+
+MIXER_SIZES = {   # width, heads, kv heads, head size, experts, top, expert ff, dense ff, window
+    "s": (1024, 8, 2, 128, 8, 2, 1024, 4096, 512),
+    "m": (2048, 16, 4, 128, 8, 2, 2048, 8192, 1024),
+    "l": (4096, 32, 8, 128, 8, 2, 4096, 14336, 1024),
+}
+
+
+def run_mixer_compare(a) -> int:
+    """One JSON line per (model, size): prompt tokens/s of the prefill steps and generated
+    tokens/s of `--steps` decode steps, `--batch-per-gpu` sequences of `--prompt-len` tokens.
+    Both models run through the same synchronous engine path (scheduler, paged cache, runner)."""
+    import torch
+
+    sys.path.insert(0, ROOT)
+    from butterfly_amd.config import EngineConfig, ModelConfig
+    from butterfly_amd.engine.engine import LLMEngine
+    from butterfly_amd.engine.sampler import SamplingParams
+
+    dev = "cuda" if torch.cuda.is_available() else "cpu"
+    B, P, K, Wm = a.batch_per_gpu, a.prompt_len, a.steps, a.warmup
+    results = []
+    for size in a.mixer_compare.split(","):
+        W, H, G, D, E, top, eff, dff, win = MIXER_SIZES[size]
+        attn = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "rot": {"dims": D // 2, "base": 1e6},
+                "scale": D ** -0.5, "mask": {"size": win, "keep_first": 4}}
+        gla = {"heads": H, "dim": D, "vdim": D, "tau": 16.0}
+        moe = {"kind": "moe", "expert": {"ff": eff, "limit": 7.0}, "router": {"experts": E, "top": top}}
+        nes = ModelConfig.from_nesizen({"architecture": "Nesizen", "vocab": 32000, "width": W, "streams": 2,
+                                        "norm": {"eps": 1e-6}, "layers": [
+                                            {"type": "gla", "mixer": gla, "mlp": {"kind": "dense", "ff": dff}},
+                                            {"type": "attention", "mixer": attn, "mlp": moe},
+                                            {"type": "attention", "mixer": dict(attn, kv_from=1), "mlp": moe},
+                                            {"type": "gla", "mixer": gla, "mlp": moe}]}, name=f"nesizen-{size}")
+        mix = ModelConfig(name=f"mixtral-{size}", arch="mixtral", vocab_size=32000, hidden_size=W,
+                          intermediate_size=eff, num_layers=4, num_heads=H, num_kv_heads=G, head_dim=D,
+                          max_position=32768, rope_theta=1e6, num_experts=E, experts_per_token=top, init_std=0.05)
+        for cfg in (nes, mix):
+            ecfg = EngineConfig(max_batch=B, max_seq_len=P + K + Wm + 8, max_prefill_tokens=8192,
+                                kv_cache_tokens=B * (P + K + Wm + 40), use_graphs=not a.no_graphs,
+                                async_decode=False, prefix_caching=False,
+                                graph_batch_sizes=sorted({1, 8, 16, 32, 64, B}))
+            eng = LLMEngine(cfg, engine_cfg=ecfg, device=dev)
+            g = torch.Generator().manual_seed(0)
+            prompts = [torch.randint(1, cfg.vocab_size, (P,), generator=g).tolist() for _ in range(B)]
+            params = SamplingParams(max_tokens=K + Wm + 2, ignore_eos=True)
+
+            def sync():
+                if dev == "cuda":
+                    torch.cuda.synchronize()
+
+            def one_round():
+                for p in prompts:
+                    eng.add_request(p, params)
+                sync()
+                t0 = time.perf_counter()
+                while eng.scheduler.num_waiting or any(len(r.output) == 0 for r in eng.requests.values() if not r.finished):
+                    eng.step()
+                sync()
+                t_pre = time.perf_counter() - t0
+                for _ in range(Wm):
+                    eng.step()
+                sync()
+                t0 = time.perf_counter()
+                for _ in range(K):
+                    eng.step()
+                sync()
+                t_dec = time.perf_counter() - t0
+                while eng.has_unfinished():
+                    eng.step()
+                eng.requests.clear()
+                return t_pre, t_dec
+
+            one_round()                      # warm-up: workspaces, graph capture
+            t_pre, t_dec = one_round()
+            line = {"model": cfg.name, "arch": cfg.arch, "width": W, "layers": 4, "batch": B, "prompt_len": P,
+                    "prefill_tokens_per_s": round(B * P / t_pre, 1), "decode_tokens_per_s": round(B * K / t_dec, 1),
+                    "decode_ms_per_step": round(1e3 * t_dec / K, 3), "dtype": "bf16" if dev == "cuda" else "fp32",
+                    "data": "synthetic", "params_m": round(cfg.param_count() / 1e6, 1)}
+            print(json.dumps(line), flush=True)
+            results.append(line)
+            eng.close()
+            del eng
+            if dev == "cuda":
+                torch.cuda.empty_cache()
+    if a.out:
+        with open(a.out, "w") as f:
+            json.dump(results, f, indent=1)
+    return 0
 
 
 def run(a) -> int:

@@ -39,6 +39,11 @@ from ..parallel.comm import Communicator
 from .shard import LocalDims, Shard
 from .transformer import LogicalParam, _name_seed
 
+def _pad128(n: int) -> int:
+    """Fused projections carry zero rows up to a multiple of 128 (the MFMA GEMMs' N tiling)."""
+    return (n + 127) // 128 * 128
+
+
 NORM_OFFSET = 1.0       # norm weights are stored around zero
 GLU_ALPHA = 1.702       # expert activation g * sigmoid(alpha g)
 
@@ -103,7 +108,7 @@ class NesizenLM:
             if sp["type"] == "attention":
                 G = sp["kv_heads"]
                 own = sp["kv_from"] is None
-                p[pre + "qkv"] = z(H * D + (G * (D + Dv) if own else 0), W)
+                p[pre + "qkv"] = z(_pad128(H * D + (G * (D + Dv) if own else 0)), W)
                 p[pre + "sink"] = f(H)
                 n = sp["rot_dims"] // 2
                 i = torch.arange(n, dtype=torch.float64)
@@ -135,7 +140,7 @@ class NesizenLM:
         W, H, D, Dv = self.cfg.hidden_size, sp["heads"], sp["dim"], sp["vdim"]
         pre = f"l{sp['index']}."
         sp["decay_rank"] = int(rank)
-        self.p[pre + "qkvga"] = torch.zeros(2 * H * D + 2 * H * Dv + rank, W, dtype=self.dtype, device=self.device)
+        self.p[pre + "qkvga"] = torch.zeros(_pad128(2 * H * D + 2 * H * Dv + rank), W, dtype=self.dtype, device=self.device)
         self.p[pre + "a2"] = torch.zeros(H * D, rank, dtype=self.dtype, device=self.device)
 
     def set_decay_ranks(self, shapes: dict) -> None:
@@ -185,7 +190,7 @@ class NesizenLM:
                 add(L + "mix.q", qkv[:H * D])
                 if sp["kv_from"] is None:
                     add(L + "mix.k", qkv[H * D:H * D + G * D])
-                    add(L + "mix.v", qkv[H * D + G * D:])
+                    add(L + "mix.v", qkv[H * D + G * D:H * D + G * D + G * sp["vdim"]])
                 add(L + "mix.sink", p[pre + "sink"], "sink")
             else:
                 fz, r = p[pre + "qkvga"], sp["decay_rank"]
@@ -345,7 +350,7 @@ class NesizenLM:
         q = qkv[:, :H * D].view(T, H, D)
         if sp["kv_from"] is None:
             k = qkv[:, H * D:H * D + G * D].view(T, G, D)
-            v = qkv[:, H * D + G * D:].view(T, G, Dv)
+            v = qkv[:, H * D + G * D:H * D + G * (D + Dv)].view(T, G, Dv)
             ops.rope_partial_kv(q, k, v, fb.positions, self.p[pre + "inv_freq"], fb.slots, kc, vc)
         else:
             ops.rope_partial_kv(q, None, None, fb.positions, self.p[pre + "inv_freq"])

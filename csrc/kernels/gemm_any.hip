@@ -272,6 +272,181 @@ __global__ __launch_bounds__(64) void moe_route_scores_kernel(const T* __restric
     for (int k = 0; k < top_k; ++k) w[(long)t * top_k + k] /= sum;
 }
 
+// ---------------------------------------------------------------------------------------
+// bf16 tile core on the matrix pipe: the same 64 x 64 output tile and the same callers, but the
+// operands are staged as bf16 (64-deep K step, 16-byte row segments, zero filled outside the
+// problem) and each of the 4 waves owns a 32 x 32 quadrant as 2 x 2 MFMA 16x16x32 tiles. The K
+// steps are accumulated in order, so a row's result does not depend on the rest of the batch.
+// ---------------------------------------------------------------------------------------
+constexpr int MK = 64, MLD = MK + 8;      // LDS row pitch 144 B: 16-byte aligned, off the bank stride
+
+struct RowRef {
+  const bf16* p;   // nullptr: a row of zeros
+  float s;         // the row is multiplied by s and rounded to bf16 (1: as stored)
+};
+
+__device__ __forceinline__ bf16x8 load_row8(const RowRef r, int k, int K) {
+  bf16x8 v;
+  if (r.p == nullptr || k >= K) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (bf16)0.f;
+    return v;
+  }
+  if (k + 8 <= K && (reinterpret_cast<uintptr_t>(r.p + k) & 15) == 0) {
+    v = *reinterpret_cast<const bf16x8*>(r.p + k);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (k + j < K) ? r.p[k + j] : (bf16)0.f;
+  }
+  if (r.s != 1.f) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (bf16)((float)v[j] * r.s);
+  }
+  return v;
+}
+
+// acc[tn][tm][i] += sum_k X(m, k) W(n, k) with m = 32 * (wave >> 1) + 16 tm + (lane & 15) and
+// n = 32 * (wave & 1) + 16 tn + 4 * (lane >> 4) + i inside the tile; rowX(r) / rowW(c) give the
+// r-th X row / c-th W row of the tile.
+template <typename FX, typename FW>
+__device__ __forceinline__ void tile_mac_mfma(f32x4 (&acc)[2][2], FX rowX, FW rowW, int K, bf16 (*Xs)[MLD],
+                                              bf16 (*Ws)[MLD]) {
+  const int tid = threadIdx.x;
+  const int lr = tid >> 2, lk = (tid & 3) * 16;        // staging: row lr, k lk .. lk + 15
+  const RowRef rx = rowX(lr), rw = rowW(lr);
+  const int wave = tid >> 6, lane = tid & 63;
+  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32, r = lane & 15, g = lane >> 4;
+  bf16x8 x0 = load_row8(rx, lk, K), x1 = load_row8(rx, lk + 8, K);
+  bf16x8 w0 = load_row8(rw, lk, K), w1 = load_row8(rw, lk + 8, K);
+  for (int k0 = 0; k0 < K; k0 += MK) {
+    *reinterpret_cast<bf16x8*>(&Xs[lr][lk]) = x0;
+    *reinterpret_cast<bf16x8*>(&Xs[lr][lk + 8]) = x1;
+    *reinterpret_cast<bf16x8*>(&Ws[lr][lk]) = w0;
+    *reinterpret_cast<bf16x8*>(&Ws[lr][lk + 8]) = w1;
+    __syncthreads();
+    if (k0 + MK < K) {          // the next K step's segments travel while this one multiplies
+      x0 = load_row8(rx, k0 + MK + lk, K);
+      x1 = load_row8(rx, k0 + MK + lk + 8, K);
+      w0 = load_row8(rw, k0 + MK + lk, K);
+      w1 = load_row8(rw, k0 + MK + lk + 8, K);
+    }
+#pragma unroll
+    for (int ks = 0; ks < MK; ks += 32) {
+      bf16x8 xf[2], wf[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        xf[t] = *reinterpret_cast<const bf16x8*>(&Xs[wm + 16 * t + r][ks + 8 * g]);
+        wf[t] = *reinterpret_cast<const bf16x8*>(&Ws[wn + 16 * t + r][ks + 8 * g]);
+      }
+#pragma unroll
+      for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < 2; ++tm) acc[tn][tm] = mfma16(wf[tn], xf[tm], acc[tn][tm]);
+    }
+    __syncthreads();
+  }
+}
+
+// f(m, n, value) over this lane's 16 results of the tile
+template <typename F>
+__device__ __forceinline__ void tile_each(const f32x4 (&acc)[2][2], F f) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+#pragma unroll
+  for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) f(wm + 16 * tm + (lane & 15), wn + 16 * tn + 4 * (lane >> 4) + i, acc[tn][tm][i]);
+}
+
+#define BFLY_ZERO_ACC(a)                                   \
+  f32x4 a[2][2];                                           \
+  _Pragma("unroll") for (int _i = 0; _i < 2; ++_i)         \
+      _Pragma("unroll") for (int _j = 0; _j < 2; ++_j) a[_i][_j] = f32x4{0.f, 0.f, 0.f, 0.f}
+
+template <typename TO>
+__global__ __launch_bounds__(256) void gemm_any_mfma_kernel(const bf16* __restrict__ x, long ldx,
+                                                            const bf16* __restrict__ w, long ldw,
+                                                            const bf16* __restrict__ bias, TO* __restrict__ out,
+                                                            long ldo, int M, int N, int K, int act) {
+  __shared__ __attribute__((aligned(16))) bf16 Xs[TM][MLD], Ws[TN][MLD];
+  const int row0 = blockIdx.y * TM, col0 = blockIdx.x * TN;
+  BFLY_ZERO_ACC(acc);
+  tile_mac_mfma(
+      acc, [&](int r) { return RowRef{row0 + r < M ? x + (long)(row0 + r) * ldx : nullptr, 1.f}; },
+      [&](int c) { return RowRef{col0 + c < N ? w + (long)(col0 + c) * ldw : nullptr, 1.f}; }, K, Xs, Ws);
+  tile_each(acc, [&](int m, int n, float v) {
+    const int r = row0 + m, c = col0 + n;
+    if (r >= M || c >= N) return;
+    if (bias) v += (float)bias[c];
+    if (act == ACT_RELU2) { v = fmaxf(v, 0.f); v = v * v; }
+    out[(long)r * ldo + c] = (TO)v;
+  });
+}
+
+__global__ __launch_bounds__(256) void moe_glu_up_mfma_kernel(const bf16* __restrict__ x, long ldx,
+                                                              const float* __restrict__ topk_w, int Kc,
+                                                              const int* __restrict__ perm,
+                                                              const int* __restrict__ offsets_e,
+                                                              const int* __restrict__ tiles,
+                                                              const int* __restrict__ ntiles,
+                                                              const bf16* __restrict__ gu_w, float limit, float alpha,
+                                                              bf16* __restrict__ hmid, int Hd, int F) {
+  if ((int)blockIdx.y >= ntiles[0]) return;
+  __shared__ __attribute__((aligned(16))) bf16 Xs[TM][MLD], Ws[TN][MLD];
+  const int e = tiles[2 * blockIdx.y], r0 = tiles[2 * blockIdx.y + 1];
+  const int rend = offsets_e[e + 1];
+  const int col0 = blockIdx.x * TN;
+  const bf16* wg = gu_w + (long)e * 2 * F * Hd;
+  const bf16* wu = wg + (long)F * Hd;
+  // the expert's input row: the token row times its routing score, rounded to bf16
+  auto rowX = [&](int r) {
+    const int p = r0 + r < rend ? perm[r0 + r] : -1;
+    return p < 0 ? RowRef{nullptr, 1.f} : RowRef{x + (long)(p / Kc) * ldx, topk_w[p]};
+  };
+  BFLY_ZERO_ACC(g);
+  BFLY_ZERO_ACC(u);
+  tile_mac_mfma(g, rowX, [&](int c) { return RowRef{col0 + c < F ? wg + (long)(col0 + c) * Hd : nullptr, 1.f}; }, Hd, Xs, Ws);
+  tile_mac_mfma(u, rowX, [&](int c) { return RowRef{col0 + c < F ? wu + (long)(col0 + c) * Hd : nullptr, 1.f}; }, Hd, Xs, Ws);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+#pragma unroll
+  for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = r0 + wm + 16 * tm + (lane & 15), c = col0 + wn + 16 * tn + 4 * (lane >> 4) + i;
+        if (r >= rend || c >= F) continue;
+        const float gg = fminf(g[tn][tm][i], limit);
+        const float uu = fminf(fmaxf(u[tn][tm][i], -limit), limit);
+        hmid[(long)r * F + c] = (bf16)(gg / (1.f + expf(-alpha * gg)) * (uu + 1.f));
+      }
+}
+
+__global__ __launch_bounds__(256) void moe_down_mfma_kernel(const bf16* __restrict__ hmid, const int* __restrict__ perm,
+                                                            const int* __restrict__ offsets_e,
+                                                            const int* __restrict__ tiles,
+                                                            const int* __restrict__ ntiles,
+                                                            const bf16* __restrict__ down_w, float* __restrict__ y,
+                                                            int Hd, int F) {
+  if ((int)blockIdx.y >= ntiles[0]) return;
+  __shared__ __attribute__((aligned(16))) bf16 Xs[TM][MLD], Ws[TN][MLD];
+  const int e = tiles[2 * blockIdx.y], r0 = tiles[2 * blockIdx.y + 1];
+  const int rend = offsets_e[e + 1];
+  const int col0 = blockIdx.x * TN;
+  const bf16* wd = down_w + (long)e * Hd * F;
+  BFLY_ZERO_ACC(acc);
+  tile_mac_mfma(
+      acc, [&](int r) { return RowRef{r0 + r < rend ? hmid + (long)(r0 + r) * F : nullptr, 1.f}; },
+      [&](int c) { return RowRef{col0 + c < Hd ? wd + (long)(col0 + c) * F : nullptr, 1.f}; }, F, Xs, Ws);
+  tile_each(acc, [&](int m, int n, float v) {
+    const int r = r0 + m, c = col0 + n;
+    if (r < rend && c < Hd) y[(long)perm[r] * Hd + c] = v;
+  });
+}
+
 inline int ew_blocks(long n) { return (int)std::min<long>(4096, std::max<long>(1, (n + 255) / 256)); }
 
 }  // namespace
@@ -284,11 +459,11 @@ void launch_gemm_any(const void* x, long ldx, const void* w, long ldw, const voi
     gemm_any_kernel<float, float><<<grid, 256, 0, s>>>((const float*)x, ldx, (const float*)w, ldw, (const float*)bias,
                                                        (float*)out, ldo, M, N, K, act);
   else if (out_f32)
-    gemm_any_kernel<bf16, float><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
-                                                      (float*)out, ldo, M, N, K, act);
+    gemm_any_mfma_kernel<float><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
+                                                     (float*)out, ldo, M, N, K, act);
   else
-    gemm_any_kernel<bf16, bf16><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
-                                                     (bf16*)out, ldo, M, N, K, act);
+    gemm_any_mfma_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
+                                                    (bf16*)out, ldo, M, N, K, act);
 }
 
 void launch_relu2(void* x, long n, bool f32, hipStream_t s) {
@@ -322,8 +497,8 @@ void launch_moe_glu_up(const void* x, long ldx, const float* topk_w, int K, cons
     moe_glu_up_kernel<float><<<grid, 256, 0, s>>>((const float*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
                                                   (const float*)gate_up_w, limit, alpha, (float*)hmid, Hd, F);
   else
-    moe_glu_up_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
-                                                 (const bf16*)gate_up_w, limit, alpha, (bf16*)hmid, Hd, F);
+    moe_glu_up_mfma_kernel<<<grid, 256, 0, s>>>((const bf16*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
+                                                (const bf16*)gate_up_w, limit, alpha, (bf16*)hmid, Hd, F);
 }
 
 void launch_moe_down(const void* hmid, const int* perm, const int* offsets, const int* tiles, const int* ntiles,
@@ -333,8 +508,8 @@ void launch_moe_down(const void* hmid, const int* perm, const int* offsets, cons
     moe_down_kernel<float><<<grid, 256, 0, s>>>((const float*)hmid, perm, offsets, tiles, ntiles,
                                                 (const float*)down_w, y, Hd, F);
   else
-    moe_down_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)hmid, perm, offsets, tiles, ntiles, (const bf16*)down_w, y,
-                                               Hd, F);
+    moe_down_mfma_kernel<<<grid, 256, 0, s>>>((const bf16*)hmid, perm, offsets, tiles, ntiles, (const bf16*)down_w, y,
+                                              Hd, F);
 }
 
 void launch_moe_sum(const float* y, int K, void* out, int T, int Hd, bool f32, hipStream_t s) {
