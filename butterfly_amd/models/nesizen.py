@@ -263,7 +263,7 @@ class NesizenLM:
         return sum(4 * sp["heads"] * sp["dim"] * sp["vdim"] for sp in self.specs if sp["type"] == "gla")
 
     def allocate_kv_cache(self, num_blocks: int, block_size: int, dtype: Optional[torch.dtype] = None) -> list:
-        """One (K [blocks, G, BS, D], V [blocks, G, BS, Dv]) pair per attention layer that has its
+        """One (K [blocks, G, BS, D], V [blocks, G, Dv, BS]) pair per attention layer that has its
         own keys, in layer order (`cache_index` maps a layer to its pair)."""
         dt = dtype or self.dtype
         if dt != self.dtype:
@@ -273,7 +273,7 @@ class NesizenLM:
             if sp["type"] == "attention" and sp["kv_from"] is None:
                 G = sp["kv_heads"]
                 caches.append((torch.zeros(num_blocks, G, block_size, sp["dim"], dtype=dt, device=self.device),
-                               torch.zeros(num_blocks, G, block_size, sp["vdim"], dtype=dt, device=self.device)))
+                               torch.zeros(num_blocks, G, sp["vdim"], block_size, dtype=dt, device=self.device)))
         return caches
 
     def allocate_state(self, num_slots: int) -> list:

@@ -794,7 +794,8 @@ def hc_final(xs, norm_w, eps: float, offset: float, idx, out_dtype):
 def rope_partial_kv(q, k, v, positions, inv_freq, slots=None, k_cache=None, v_cache=None):
     """Interleaved-pair rotary on the first 2 * len(inv_freq) dims of the q [T, H, D] and
     k [T, G, D] heads, in place, and the append of k, v [T, G, Dv] to the paged caches
-    K [blocks, G, BS, D], V [blocks, G, BS, Dv]. k None: q only."""
+    K [blocks, G, BS, D], V [blocks, G, Dv, BS] (V transposed, as the framework's other caches).
+    k None: q only."""
     if not _gpu(q):
         return ref.rope_partial_kv(q, k, v, positions, inv_freq, slots, k_cache, v_cache)
     torch.ops.bfly.rope_partial_kv(q, k, v, positions, inv_freq, slots, k_cache, v_cache)
@@ -816,10 +817,10 @@ def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale: flo
     if not _gpu(q):
         return ref.attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, window, keep_first, sink, out)
     if out is None:
-        out = _empty(q.shape[0], q.shape[1], v_cache.shape[3], dtype=q.dtype, device=q.device)
+        out = _empty(q.shape[0], q.shape[1], v_cache.shape[2], dtype=q.dtype, device=q.device)
     if row_map is None:
         row_map = row_seq(row_cu, q.shape[0])
-    torch.ops.bfly.attn_window_paged(q, k_cache, v_cache, tables, row_map, positions, float(scale), int(window),
+    torch.ops.bfly.attn_window_paged(q, k_cache, v_cache, tables, row_map, row_cu, positions, float(scale), int(window),
                                      int(keep_first), sink, out)
     return out
 

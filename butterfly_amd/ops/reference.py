@@ -539,8 +539,8 @@ def ep_combine(back, slot):
 # Heterogeneous-stack mechanisms: offset-weight norms over parallel residual streams
 # (hyper-connections), partial interleaved rotary, windowed attention with kept first tokens
 # and a sink logit, gated linear attention with a per-sequence recurrent state, sigmoid-scored
-# MoE with clamped GLU experts. Caches of these mixers: K [blocks, G, BS, D], V [blocks, G, BS, Dv]
-# (both row layouts), recurrent state [slots, H, D, Dv] f32.
+# MoE with clamped GLU experts. Caches of these mixers: K [blocks, G, BS, D], V [blocks, G, Dv, BS]
+# (V transposed), recurrent state [slots, H, D, Dv] f32.
 # ---------------------------------------------------------------------------------------
 def linear_act(x, w, bias=None, act="none", out_dtype=None):
     """y = act(x w^T + bias), f32 accumulation; act: none | relu2 (relu squared)."""
@@ -597,7 +597,7 @@ def rope_partial_kv(q, k, v, positions, inv_freq, slots, k_cache, v_cache):
         ok = slots >= 0
         sl = slots[ok].long()
         k_cache[sl // bs, :, sl % bs] = k[ok].to(k_cache.dtype)
-        v_cache[sl // bs, :, sl % bs] = v[ok].to(v_cache.dtype)
+        v_cache[sl // bs, :, :, sl % bs] = v[ok].to(v_cache.dtype)
     return q
 
 
@@ -606,7 +606,7 @@ def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, win
     keys j <= p of tables[s] with p - j < window or j < keep_first; the softmax denominator
     also holds exp(sink[h])."""
     T, H, D = q.shape
-    G, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    G, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
     o = torch.zeros(T, H, Dv, dtype=torch.float32, device=q.device)
     cu = row_cu.tolist()
     pos = positions.tolist()
@@ -617,7 +617,7 @@ def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, win
         nb = pmax // bs + 1
         blk = tables[s, :nb].long()
         K = k_cache[blk].float().permute(1, 0, 2, 3).reshape(G, nb * bs, D)
-        V = v_cache[blk].float().permute(1, 0, 2, 3).reshape(G, nb * bs, Dv)
+        V = v_cache[blk].float().permute(1, 0, 3, 2).reshape(G, nb * bs, Dv)
         j = torch.arange(nb * bs, device=q.device)[None, :]
         p = positions[cu[s]:cu[s + 1]].long()[:, None]
         ok = (j <= p) & ((p - j < window) | (j < keep_first))

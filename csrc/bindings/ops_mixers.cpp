@@ -121,9 +121,9 @@ void rope_partial_kv(Tensor& q, const optional<Tensor>& k, const optional<Tensor
     TORCH_CHECK(K.size(0) == T && V.size(0) == T && K.size(2) == D && V.size(1) == G && slots->numel() == T,
                 "rope_partial_kv: k / v shapes");
     TORCH_CHECK(KC.dim() == 4 && VC.dim() == 4 && KC.is_contiguous() && VC.is_contiguous() && KC.size(1) == G &&
-                    KC.size(3) == D && VC.size(0) == KC.size(0) && VC.size(1) == G && VC.size(2) == KC.size(2) &&
-                    VC.size(3) == Dv,
-                "rope_partial_kv: caches must be K [blocks, G, BS, D], V [blocks, G, BS, Dv]");
+                    KC.size(3) == D && VC.size(0) == KC.size(0) && VC.size(1) == G && VC.size(3) == KC.size(2) &&
+                    VC.size(2) == Dv,
+                "rope_partial_kv: caches must be K [blocks, G, BS, D], V [blocks, G, Dv, BS]");
     bs = KC.size(2);
     // slots are produced by the block manager for this cache: blocks * BS bounds them
     kp = K.data_ptr(); vp = V.data_ptr(); kc = KC.data_ptr(); vc = VC.data_ptr(); sp = slots->data_ptr<int>();
@@ -142,22 +142,30 @@ void row_seq(const Tensor& row_cu, Tensor& out) {
 }
 
 void attn_window_paged(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, const Tensor& tables,
-                       const Tensor& row_seq_t, const Tensor& positions, double scale, int64_t window,
-                       int64_t keep_first, const Tensor& sink, Tensor& out) {
+                       const Tensor& row_seq_t, const Tensor& row_cu, const Tensor& positions, double scale,
+                       int64_t window, int64_t keep_first, const Tensor& sink, Tensor& out) {
   CHK_GPU(q); CHK_HEADS(q); CHK_SAME(k_cache, q); CHK_SAME(v_cache, q); CHK_SAME(out, q);
   CHK_I32(tables); CHK_I32(row_seq_t); CHK_I32(positions); CHK_F32(sink);
   const int64_t T = q.size(0), H = q.size(1), D = q.size(2);
   TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.is_contiguous(),
               "attn_window_paged: caches");
-  const int64_t G = k_cache.size(1), bs = k_cache.size(2), Dv = v_cache.size(3);
-  TORCH_CHECK(k_cache.size(3) == D && v_cache.size(1) == G && v_cache.size(2) == bs && v_cache.size(0) == k_cache.size(0),
-              "attn_window_paged: cache shapes");
+  const int64_t G = k_cache.size(1), bs = k_cache.size(2), Dv = v_cache.size(2);
+  TORCH_CHECK(k_cache.size(3) == D && v_cache.size(1) == G && v_cache.size(3) == bs && v_cache.size(0) == k_cache.size(0),
+              "attn_window_paged: cache shapes K [blocks, G, BS, D], V [blocks, G, Dv, BS]");
+  CHK_I32(row_cu);
+  TORCH_CHECK(row_cu.numel() == tables.size(0) + 1, "attn_window_paged: row_cu");
   TORCH_CHECK(G > 0 && H % G == 0 && Dv <= 256 && D <= 4096, "attn_window_paged: head counts / sizes");
   TORCH_CHECK(tables.dim() == 2 && row_seq_t.numel() == T && positions.numel() == T && sink.numel() == H,
               "attn_window_paged: index shapes");
   TORCH_CHECK(out.is_contiguous() && out.dim() == 3 && out.size(0) == T && out.size(1) == H && out.size(2) == Dv,
               "attn_window_paged: out");
   TORCH_CHECK(window >= 1 && keep_first >= 0, "attn_window_paged: window >= 1, keep_first >= 0");
+  if (!is_f32(q) && bfly::launch_attn_window_mfma(q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+                                                  tables.data_ptr<int>(), (int)tables.size(1), row_cu.data_ptr<int>(),
+                                                  (int)tables.size(0), positions.data_ptr<int>(), (float)scale,
+                                                  (int)window, (int)keep_first, sink.data_ptr<float>(), out.data_ptr(),
+                                                  (int)T, (int)H, (int)G, (int)D, (int)Dv, (int)bs, cur_stream()))
+    return;
   bfly::launch_attn_window_paged(q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                  tables.data_ptr<int>(), (int)tables.size(1), row_seq_t.data_ptr<int>(),
                                  (int)tables.size(0), positions.data_ptr<int>(), (float)scale, (int)window,
@@ -264,8 +272,8 @@ TORCH_LIBRARY_FRAGMENT(bfly, m) {
   m.def("rope_partial_kv(Tensor(a!) q, Tensor(b!)? k, Tensor? v, Tensor positions, Tensor inv_freq, Tensor? slots, "
         "Tensor(c!)? k_cache, Tensor(d!)? v_cache) -> ()");
   m.def("row_seq(Tensor row_cu, Tensor(a!) out) -> ()");
-  m.def("attn_window_paged(Tensor q, Tensor k_cache, Tensor v_cache, Tensor tables, Tensor row_seq, Tensor positions, "
-        "float scale, int window, int keep_first, Tensor sink, Tensor(a!) out) -> ()");
+  m.def("attn_window_paged(Tensor q, Tensor k_cache, Tensor v_cache, Tensor tables, Tensor row_seq, Tensor row_cu, "
+        "Tensor positions, float scale, int window, int keep_first, Tensor sink, Tensor(a!) out) -> ()");
   m.def("gla_scan(Tensor q, Tensor k, Tensor v, Tensor z, Tensor(a!) state, Tensor state_slots, Tensor row_cu, "
         "Tensor positions, float tau, float q_scale, Tensor(b!) o) -> ()");
   m.def("gla_out(Tensor o, Tensor g, Tensor norm_w, float eps, Tensor(a!) out) -> ()");

@@ -33,7 +33,7 @@ void launch_hc_final(const float* xs, const float* norm_w, float eps, float offs
                      int R, int S, int W, bool f32, hipStream_t s);
 
 // Rotate pairs (2i, 2i+1), i < nrot, of every q and k head by positions[t] * inv_freq[i]; append
-// k / v rows to cache slot slots[t] (>= 0). k == nullptr: q only.
+// k / v rows to cache slot slots[t] (>= 0): K [blocks, G, BS, D], V [blocks, G, Dv, BS]. k == nullptr: q only.
 void launch_rope_partial_kv(void* q, long q_ld, void* k, long k_ld, const void* v, long v_ld, const int* positions,
                             const float* inv_freq, int nrot, const int* slots, void* k_cache, void* v_cache,
                             int T, int H, int G, int D, int Dv, int block_size, bool f32, hipStream_t s);
@@ -46,6 +46,13 @@ void launch_attn_window_paged(const void* q, long q_ld, const void* k_cache, con
                               int max_blocks, const int* row_seq, int nseq, const int* positions, float scale,
                               int window, int keep_first, const float* sink, void* out, int T, int H, int G, int D,
                               int Dv, int block_size, bool f32, hipStream_t s);
+
+// The MFMA form of launch_attn_window_paged over row_cu (bf16, 32-token pages, D in {32, 64, 128,
+// 256}, Dv in {32, 64, 128, 256}, 16-byte aligned q rows): false if the shape has no such form.
+bool launch_attn_window_mfma(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
+                             int max_blocks, const int* row_cu, int nseq, const int* positions, float scale, int window,
+                             int keep_first, const float* sink, void* out, int T, int H, int G, int D, int Dv,
+                             int block_size, hipStream_t s);
 
 // Gated linear attention scan over packed rows (see ops.gla_scan). Returns < 0 if D > 256.
 int launch_gla_scan(const void* q, long q_ld, const void* k, long k_ld, const void* v, long v_ld, const void* z,

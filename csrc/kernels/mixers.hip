@@ -1,8 +1,9 @@
 // Sequence mixers for heterogeneous layer stacks, generic in head count, head sizes and element
 // type (bf16 or f32 activations / caches; scores, softmax, angles, decays and state are f32):
 //   rope_partial_kv_kernel    interleaved-pair rotary on the first 2 * nrot dims of q / k heads,
-//                             fused with the paged append of k and v (row layouts
-//                             K [blocks, G, BS, D], V [blocks, G, BS, Dv])
+//                             fused with the paged append of k and v
+//                             (K [blocks, G, BS, D] rows, V [blocks, G, Dv, BS] transposed: a
+//                             page's keys are contiguous for the P V operand)
 //   attn_window_paged_kernel  attention of packed rows over the paged cache: causal sliding
 //                             window plus the always-visible first `keep_first` positions, and a
 //                             per-head sink logit that only enters the softmax denominator
@@ -55,7 +56,7 @@ __global__ __launch_bounds__(256) void rope_partial_kv_kernel(T* __restrict__ q,
   }
   for (int i = threadIdx.x; i < G * Dv; i += blockDim.x) {
     const int g = i / Dv, d = i % Dv;
-    v_cache[((blk * G + g) * bs + off) * Dv + d] = v[t * v_ld + i];
+    v_cache[((blk * G + g) * Dv + d) * bs + off] = v[t * v_ld + i];
   }
 }
 
@@ -98,11 +99,12 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
   for (int i0 = 0; i0 < total; i0 += 64) {
     const int i = i0 + lane;
     float sc = -INFINITY;
-    long kv_row = 0;
+    long kv_row = 0;      // index of V^T[0][key] of this lane's key
     if (i < total) {
       const int j = i < n1 ? i : lo + (i - n1);
-      kv_row = ((long)tab[j / bs] * G + g) * bs + (j % bs);
-      const T* kr = k_cache + kv_row * D;
+      const long pg = (long)tab[j / bs] * G + g;
+      kv_row = pg * Dv * bs + (j % bs);
+      const T* kr = k_cache + (pg * bs + (j % bs)) * D;
       float a = 0.f;
       for (int d = 0; d < D; ++d) a = fmaf(sq[d], (float)kr[d], a);
       sc = a * scale;
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
       const int d = lane + 64 * c;
       if (d >= Dv) break;
       float a = acc[c] * corr;
-      for (int x = 0; x < cnt; ++x) a = fmaf(sp[x], (float)v_cache[sj[x] * Dv + d], a);
+      for (int x = 0; x < cnt; ++x) a = fmaf(sp[x], (float)v_cache[sj[x] + (long)d * bs], a);
       acc[c] = a;
     }
   }
@@ -131,6 +133,121 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
   for (int c = 0; c < kMaxDvLane; ++c) {
     const int d = lane + 64 * c;
     if (d < Dv) out[(t * H + h) * Dv + d] = (T)(acc[c] * inv);
+  }
+}
+
+// MFMA form for bf16 with 32-token pages, D = 32 DS, Dv = 16 DVT: one wave per 16 consecutive
+// rows of a sequence and one query head, no LDS. Per page: S^T = K Q^T (16x16x32 tiles, K rows
+// read as 16-byte segments straight from the page), masks and an online softmax in f32 (the four
+// lanes that share a query row combine by shuffles), then O^T += V^T P with the page's keys as
+// the MFMA k index in the order the score tiles leave them (keys 4g..4g+3 and 16+4g..16+4g+3 in
+// lane group g), which the transposed V page serves with two 8-byte reads. The softmax is
+// seeded with the sink (m = sink, l = 1). Pages outside the window and the kept prefix are
+// skipped; the per-element mask settles the edges.
+template <int DS, int DVT>
+__global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __restrict__ q, long q_ld,
+                                                               const bf16* __restrict__ k_cache,
+                                                               const bf16* __restrict__ v_cache,
+                                                               const int* __restrict__ tables, int max_blocks,
+                                                               const int* __restrict__ row_cu, int nseq,
+                                                               const int* __restrict__ positions, float scale,
+                                                               int window, int keep_first,
+                                                               const float* __restrict__ sink,
+                                                               bf16* __restrict__ out, int H, int G) {
+  constexpr int D = 32 * DS, Dv = 16 * DVT, BS = 32;
+  const int lane = threadIdx.x & 63;
+  int tile = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int h = blockIdx.y, g = h / (H / G);
+  int s = 0, row0 = 0, rend = 0;
+  for (; s < nseq; ++s) {
+    const int a = row_cu[s], b = row_cu[s + 1];
+    const int nt = (b - a + 15) >> 4;
+    if (tile < nt) { row0 = a + 16 * tile; rend = b; break; }
+    tile -= nt;
+  }
+  if (s >= nseq) return;
+  const int qr = lane & 15, gg = lane >> 4;
+  const bool rv = row0 + qr < rend;
+  const long row = rv ? row0 + qr : row0;
+  const int p = rv ? positions[row] : -1;
+  int pmin = rv ? p : 0x7fffffff, pmax = p;
+#pragma unroll
+  for (int o = 1; o < 16; o <<= 1) {
+    pmin = min(pmin, __shfl_xor(pmin, o, 64));
+    pmax = max(pmax, __shfl_xor(pmax, o, 64));
+  }
+  bf16x8 qf[DS];
+#pragma unroll
+  for (int ds = 0; ds < DS; ++ds)
+    qf[ds] = *reinterpret_cast<const bf16x8*>(q + row * q_ld + (long)h * D + 32 * ds + 8 * gg);
+  const int* tab = tables + (long)s * max_blocks;
+  float m = sink[h], l = 1.f;
+  f32x4 o[DVT];
+#pragma unroll
+  for (int t = 0; t < DVT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int kp = (min(keep_first, pmax + 1) + BS - 1) / BS;          // pages of the kept prefix
+  const int wp0 = max(max(0, pmin - window + 1) / BS, kp), wp1 = pmax / BS;
+  for (int pg = 0; pg <= wp1; pg = (pg + 1 == kp && wp0 > kp) ? wp0 : pg + 1) {
+    if (pg >= kp && pg < wp0) { pg = wp0 - 1; continue; }
+    const long blk = (long)tab[pg] * G + g;
+    const bf16* Kp = k_cache + blk * BS * D;
+    const bf16* Vp = v_cache + blk * Dv * BS;
+    f32x4 st[2];
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) {
+      st[kh] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ds = 0; ds < DS; ++ds) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Kp + (long)(16 * kh + qr) * D + 32 * ds + 8 * gg);
+        st[kh] = mfma16(kf, qf[ds], st[kh]);
+      }
+    }
+    float sc[8], mx = -INFINITY;
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int j = pg * BS + 16 * kh + 4 * gg + i;
+        const bool ok = j <= p && (p - j < window || j < keep_first);
+        sc[4 * kh + i] = ok ? st[kh][i] * scale : -INFINITY;
+        mx = fmaxf(mx, sc[4 * kh + i]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mn = fmaxf(m, mx);
+    const float corr = __expf(m - mn);
+    float rs = 0.f;
+    bf16x8 pb;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float pe = __expf(sc[e] - mn);      // exp(-inf) = 0 for masked keys
+      rs += pe;
+      pb[e] = (bf16)pe;
+    }
+    rs += __shfl_xor(rs, 16, 64);
+    rs += __shfl_xor(rs, 32, 64);
+    l = l * corr + rs;
+    m = mn;
+#pragma unroll
+    for (int t = 0; t < DVT; ++t) {
+      const bf16* vr = Vp + (long)(16 * t + qr) * BS + 4 * gg;
+      const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vr);
+      const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vr + 16);
+      const bf16x8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[t][i] *= corr;
+      o[t] = mfma16(vf, pb, o[t]);
+    }
+  }
+  if (!rv) return;
+  const float inv = 1.f / l;
+  bf16* orow = out + (row * H + h) * Dv;
+#pragma unroll
+  for (int t = 0; t < DVT; ++t) {
+    bf16x4 w;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (bf16)(o[t][i] * inv);
+    *reinterpret_cast<bf16x4*>(orow + 16 * t + 4 * gg) = w;
   }
 }
 
@@ -248,6 +365,44 @@ void launch_rope_partial_kv(void* q, long q_ld, void* k, long k_ld, const void* 
 void launch_row_seq(const int* row_cu, int nseq, int* row_seq, int T, hipStream_t s) {
   if (T <= 0) return;
   row_seq_kernel<<<(T + 255) / 256, 256, 0, s>>>(row_cu, nseq, row_seq, T);
+}
+
+template <int DS>
+static bool attn_mfma_dv(const bf16* q, long q_ld, const bf16* kc, const bf16* vc, const int* tables, int max_blocks,
+                         const int* row_cu, int nseq, const int* positions, float scale, int window, int keep_first,
+                         const float* sink, bf16* out, int T, int H, int G, int Dv, hipStream_t s) {
+  // every sequence adds at most one partly filled 16-row tile
+  dim3 grid(((T + 15) / 16 + nseq + 3) / 4, H);
+#define BFLY_ATT(DVT)                                                                                            \
+  attn_window_mfma_kernel<DS, DVT><<<grid, 256, 0, s>>>(q, q_ld, kc, vc, tables, max_blocks, row_cu, nseq, positions, \
+                                                        scale, window, keep_first, sink, out, H, G)
+  switch (Dv) {
+    case 32: BFLY_ATT(2); return true;
+    case 64: BFLY_ATT(4); return true;
+    case 128: BFLY_ATT(8); return true;
+    case 256: BFLY_ATT(16); return true;
+    default: return false;
+  }
+#undef BFLY_ATT
+}
+
+bool launch_attn_window_mfma(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
+                             int max_blocks, const int* row_cu, int nseq, const int* positions, float scale, int window,
+                             int keep_first, const float* sink, void* out, int T, int H, int G, int D, int Dv,
+                             int block_size, hipStream_t s) {
+  if (block_size != 32 || (q_ld & 7) || (reinterpret_cast<uintptr_t>(q) & 15)) return false;
+  if (T <= 0) return true;
+#define BFLY_ATTD(DS)                                                                                          \
+  return attn_mfma_dv<DS>((const bf16*)q, q_ld, (const bf16*)k_cache, (const bf16*)v_cache, tables, max_blocks, row_cu, \
+                          nseq, positions, scale, window, keep_first, sink, (bf16*)out, T, H, G, Dv, s)
+  switch (D) {
+    case 32: BFLY_ATTD(1);
+    case 64: BFLY_ATTD(2);
+    case 128: BFLY_ATTD(4);
+    case 256: BFLY_ATTD(8);
+    default: return false;
+  }
+#undef BFLY_ATTD
 }
 
 void launch_attn_window_paged(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,

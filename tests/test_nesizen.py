@@ -130,7 +130,7 @@ def test_rotary_pairs_and_append(target, D, rot):
     pos = torch.tensor([0, 1, 2, 500, 501, 77777, 3])
     slots = torch.tensor([20, 21, 22, 3, 0, 9, -1])
     inv = torch.tensor([base ** (-2.0 * i / max(rot, 1)) for i in range(rot // 2)], dtype=torch.float32)
-    kc, vc = torch.zeros(nb, G, bs, D, dtype=dt, device=dev), torch.zeros(nb, G, bs, Dv, dtype=dt, device=dev)
+    kc, vc = torch.zeros(nb, G, bs, D, dtype=dt, device=dev), torch.zeros(nb, G, Dv, bs, dtype=dt, device=dev)
     qd, kd, vd = q.to(dev, dt), k.to(dev, dt), v.to(dev, dt)
     ops.rope_partial_kv(qd, kd, vd, pos.to(torch.int32).to(dev), inv.to(dev), slots.to(torch.int32).to(dev), kc, vc)
     wq, wk = O.rotate_pairs(q, pos, rot, base), O.rotate_pairs(k, pos, rot, base)
@@ -141,7 +141,7 @@ def test_rotary_pairs_and_append(target, D, rot):
         if s < 0:
             continue
         assert (kc[s // bs, :, s % bs].cpu().to(F64) - wk[i]).abs().max() < t
-        assert (vc[s // bs, :, s % bs].cpu().to(F64) - v[i]).abs().max() < 1e-6
+        assert (vc[s // bs, :, :, s % bs].cpu().to(F64) - v[i]).abs().max() < 1e-6
     assert float(kc[[1, 3, 4]].abs().sum()) == 0 and float(vc[[1, 3, 4]].abs().sum()) == 0    # other pages untouched
 
 
@@ -152,10 +152,10 @@ def _paged(k, v, bs, perm_seed, dev, dt, extra=3):
     g = torch.Generator().manual_seed(perm_seed)
     pages = torch.randperm(nb + extra, generator=g)[:nb]
     kc = torch.full((nb + extra, G, bs, D), 9.0, dtype=dt, device=dev)       # stale values elsewhere
-    vc = torch.full((nb + extra, G, bs, v.shape[2]), -9.0, dtype=dt, device=dev)
+    vc = torch.full((nb + extra, G, v.shape[2], bs), -9.0, dtype=dt, device=dev)      # V pages are transposed
     for j in range(L):
         kc[pages[j // bs], :, j % bs] = k[j].to(dev, dt)
-        vc[pages[j // bs], :, j % bs] = v[j].to(dev, dt)
+        vc[pages[j // bs], :, :, j % bs] = v[j].to(dev, dt)
     return kc, vc, pages.to(torch.int32)
 
 
