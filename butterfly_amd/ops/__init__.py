@@ -849,9 +849,11 @@ def moe_route_scores(x, wr, top_k: int, scoring: str = "softmax", renorm: bool =
     if not _gpu(x):
         return ref.moe_route_scores(x, wr, top_k, scoring, renorm)
     T = x.shape[0]
+    # logits: a GEMM with f32 accumulation and f32 output, then one wave per token picks
+    logits = linear_act(x, wr, out_dtype=torch.float32)
     ids = _empty(T, top_k, dtype=torch.int32, device=x.device)
     w = _empty(T, top_k, dtype=torch.float32, device=x.device)
-    torch.ops.bfly.moe_route_scores(x, wr, top_k, {"softmax": 0, "sigmoid": 1}[scoring], bool(renorm), ids, w)
+    torch.ops.bfly.moe_topk_scores(logits, top_k, {"softmax": 0, "sigmoid": 1}[scoring], bool(renorm), ids, w)
     return ids, w
 
 

@@ -203,16 +203,14 @@ void gla_out(const Tensor& o, const Tensor& g, const Tensor& norm_w, double eps,
                        out.data_ptr(), (int)T, (int)H, (int)Dv, is_f32(out), cur_stream());
 }
 
-void moe_route_scores(const Tensor& x, const Tensor& wr, int64_t top_k, int64_t scoring, bool renorm, Tensor& ids,
-                      Tensor& w) {
-  CHK_GPU(x); CHK_SAME(x, wr); CHK_I32(ids); CHK_F32(w);
-  TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1 && wr.dim() == 2 && wr.is_contiguous(), "moe_route_scores: layouts");
-  const int64_t T = x.size(0), Hd = x.size(1), E = wr.size(0);
-  TORCH_CHECK(wr.size(1) == Hd && E >= 1 && E <= 1024 && top_k >= 1 && top_k <= E, "moe_route_scores: experts / top_k");
-  TORCH_CHECK(ids.numel() == T * top_k && w.numel() == T * top_k, "moe_route_scores: outputs");
-  bfly::launch_moe_route_scores(x.data_ptr(), x.stride(0), wr.data_ptr(), (int)top_k, (int)scoring, renorm,
-                                ids.data_ptr<int>(), w.data_ptr<float>(), (int)T, (int)E, (int)Hd, is_f32(x),
-                                cur_stream());
+void moe_topk_scores(const Tensor& logits, int64_t top_k, int64_t scoring, bool renorm, Tensor& ids, Tensor& w) {
+  CHK_GPU(logits); CHK_F32(logits); CHK_I32(ids); CHK_F32(w);
+  TORCH_CHECK(logits.dim() == 2, "moe_topk_scores: logits [T, E]");
+  const int64_t T = logits.size(0), E = logits.size(1);
+  TORCH_CHECK(E >= 1 && E <= 1024 && top_k >= 1 && top_k <= E, "moe_topk_scores: experts / top_k");
+  TORCH_CHECK(ids.numel() == T * top_k && w.numel() == T * top_k, "moe_topk_scores: outputs");
+  bfly::launch_moe_topk_scores(logits.data_ptr<float>(), (int)top_k, (int)scoring, renorm, ids.data_ptr<int>(),
+                               w.data_ptr<float>(), (int)T, (int)E, cur_stream());
 }
 
 int64_t moe_sort_max_tiles(int64_t TK, int64_t E) { return bfly::moe_sort_max_tiles((int)TK, (int)E); }
@@ -277,7 +275,7 @@ TORCH_LIBRARY_FRAGMENT(bfly, m) {
   m.def("gla_scan(Tensor q, Tensor k, Tensor v, Tensor z, Tensor(a!) state, Tensor state_slots, Tensor row_cu, "
         "Tensor positions, float tau, float q_scale, Tensor(b!) o) -> ()");
   m.def("gla_out(Tensor o, Tensor g, Tensor norm_w, float eps, Tensor(a!) out) -> ()");
-  m.def("moe_route_scores(Tensor x, Tensor wr, int top_k, int scoring, bool renorm, Tensor(a!) ids, Tensor(b!) w) -> ()");
+  m.def("moe_topk_scores(Tensor logits, int top_k, int scoring, bool renorm, Tensor(a!) ids, Tensor(b!) w) -> ()");
   m.def("moe_sort_max_tiles(int tk, int experts) -> int", &moe_sort_max_tiles);
   m.def("moe_glu_ffn(Tensor x, Tensor topk_ids, Tensor topk_w, Tensor gate_up_w, Tensor down_w, float limit, "
         "float alpha, Tensor(a!) work, Tensor(b!) hmid, Tensor(c!) y, Tensor(d!) out) -> ()");
@@ -296,6 +294,6 @@ TORCH_LIBRARY_IMPL(bfly, CUDA, m) {
   m.impl("attn_window_paged", &attn_window_paged);
   m.impl("gla_scan", &gla_scan);
   m.impl("gla_out", &gla_out);
-  m.impl("moe_route_scores", &moe_route_scores);
+  m.impl("moe_topk_scores", &moe_topk_scores);
   m.impl("moe_glu_ffn", &moe_glu_ffn);
 }

@@ -63,10 +63,10 @@ int launch_gla_scan(const void* q, long q_ld, const void* k, long k_ld, const vo
 void launch_gla_out(const float* o, const void* g, long g_ld, const float* norm_w, float eps, void* out, int T, int H,
                     int Dv, bool f32, hipStream_t s);
 
-// Router: f32 logits, scoring 0 softmax / 1 sigmoid, top-k (ties: lowest id), optional renorm.
-// E <= 1024.
-void launch_moe_route_scores(const void* x, long ldx, const void* wr, int top_k, int scoring, bool renorm, int* ids,
-                             float* w, int T, int E, int Hd, bool f32, hipStream_t s);
+// Router choice from f32 logits [T, E]: scoring 0 softmax / 1 sigmoid, top-k (ties: lowest id),
+// optional renorm. E <= 1024.
+void launch_moe_topk_scores(const float* logits, int top_k, int scoring, bool renorm, int* ids, float* w, int T, int E,
+                            hipStream_t s);
 // Group the T*K (token, choice) pairs by expert: perm [TK] pair indices grouped by expert,
 // offsets [E + 1], tiles [max_tiles][2] = (expert, first row) of every 64-row tile, ntiles [1].
 void launch_moe_sort(const int* ids, int TK, int E, int* perm, int* offsets, int* tiles, int* ntiles, hipStream_t s);

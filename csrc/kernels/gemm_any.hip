@@ -215,22 +215,14 @@ __global__ void moe_sum_kernel(const float* __restrict__ y, int Kc, T* __restric
   }
 }
 
-// Router scores of one token per wave: f32 logits (lanes split the hidden dim), softmax or
-// sigmoid, K rounds of arg-max over the experts (ties to the lowest id).
-template <typename T>
-__global__ __launch_bounds__(64) void moe_route_scores_kernel(const T* __restrict__ x, long ldx,
-                                                              const T* __restrict__ wr, int top_k, int scoring,
-                                                              int renorm, int* __restrict__ ids, float* __restrict__ w,
-                                                              int E, int Hd) {
+// Router choice of one token per wave from its f32 logits [E]: softmax or sigmoid scores, K rounds
+// of arg-max over the experts (ties to the lowest id).
+__global__ __launch_bounds__(64) void moe_topk_scores_kernel(const float* __restrict__ logits, int top_k, int scoring,
+                                                             int renorm, int* __restrict__ ids, float* __restrict__ w,
+                                                             int E) {
   __shared__ float sc[1024];
   const int t = blockIdx.x, lane = threadIdx.x;
-  const T* xr = x + (long)t * ldx;
-  for (int e = 0; e < E; ++e) {
-    float a = 0.f;
-    for (int k = lane; k < Hd; k += 64) a = fmaf(ldf(xr + k), ldf(wr + (long)e * Hd + k), a);
-    a = wave_sum(a);
-    if (lane == 0) sc[e] = a;
-  }
+  for (int e = lane; e < E; e += 64) sc[e] = logits[(long)t * E + e];
   __syncthreads();
   if (scoring == 0) {
     float mx = -INFINITY;
@@ -472,15 +464,10 @@ void launch_relu2(void* x, long n, bool f32, hipStream_t s) {
   else relu2_kernel<bf16><<<ew_blocks(n), 256, 0, s>>>((bf16*)x, n);
 }
 
-void launch_moe_route_scores(const void* x, long ldx, const void* wr, int top_k, int scoring, bool renorm, int* ids,
-                             float* w, int T, int E, int Hd, bool f32, hipStream_t s) {
+void launch_moe_topk_scores(const float* logits, int top_k, int scoring, bool renorm, int* ids, float* w, int T, int E,
+                            hipStream_t s) {
   if (T <= 0) return;
-  if (f32)
-    moe_route_scores_kernel<float><<<T, 64, 0, s>>>((const float*)x, ldx, (const float*)wr, top_k, scoring, renorm,
-                                                    ids, w, E, Hd);
-  else
-    moe_route_scores_kernel<bf16><<<T, 64, 0, s>>>((const bf16*)x, ldx, (const bf16*)wr, top_k, scoring, renorm, ids,
-                                                   w, E, Hd);
+  moe_topk_scores_kernel<<<T, 64, 0, s>>>(logits, top_k, scoring, renorm, ids, w, E);
 }
 
 int moe_sort_max_tiles(int TKp, int E) { return (TKp + 63) / 64 + E; }

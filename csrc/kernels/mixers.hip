@@ -294,17 +294,33 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(const T* __restrict__ q, 
     const int d = w + 4 * i;
     st[i] = (!fresh && live && d < D) ? S[(long)d * Dv + col] : 0.f;
   }
+  // the next token's operands are loaded while the current one is folded into the state
+  const bool stager = (int)threadIdx.x < D;
+  const int d0 = threadIdx.x;
+  float nz = 0.f, nk = 0.f, nq = 0.f, nv = 0.f;
+  if (stager) {
+    nz = (float)z[(long)r0 * z_ld + (long)h * D + d0];
+    nk = (float)k[(long)r0 * k_ld + (long)h * D + d0];
+    nq = (float)q[(long)r0 * q_ld + (long)h * D + d0];
+  }
+  if (live) nv = (float)v[(long)r0 * v_ld + (long)h * Dv + col];
   for (int t = r0; t < r1; ++t) {
-    if ((int)threadIdx.x < D) {
-      const int d = threadIdx.x;
-      const float zz = (float)z[(long)t * z_ld + (long)h * D + d];
+    const float zz = nz, kk = nk, qq = nq, vv = nv;
+    if (t + 1 < r1) {
+      if (stager) {
+        nz = (float)z[(long)(t + 1) * z_ld + (long)h * D + d0];
+        nk = (float)k[(long)(t + 1) * k_ld + (long)h * D + d0];
+        nq = (float)q[(long)(t + 1) * q_ld + (long)h * D + d0];
+      }
+      if (live) nv = (float)v[(long)(t + 1) * v_ld + (long)h * Dv + col];
+    }
+    if (stager) {
       // log sigmoid(z) = -softplus(-z), stable on both sides
       const float ls = zz < 0.f ? zz - log1pf(expf(zz)) : -log1pf(expf(-zz));
-      sa[d] = expf(ls * inv_tau);
-      sk[d] = (float)k[(long)t * k_ld + (long)h * D + d];
-      sq[d] = (float)q[(long)t * q_ld + (long)h * D + d] * q_scale;
+      sa[d0] = expf(ls * inv_tau);
+      sk[d0] = kk;
+      sq[d0] = qq * q_scale;
     }
-    const float vv = live ? (float)v[(long)t * v_ld + (long)h * Dv + col] : 0.f;
     __syncthreads();
     float po = 0.f;
 #pragma unroll
