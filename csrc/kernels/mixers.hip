@@ -261,29 +261,35 @@ __global__ void row_seq_kernel(const int* __restrict__ row_cu, int nseq, int* __
   row_seq[t] = s;
 }
 
-// Workgroup = (sequence, head, 64-column slice of Dv), 4 waves. Wave w keeps rows d = w, w+4, ...
-// of the slice's state in registers (NR per lane, lane = column); per token the decays, keys and
-// queries of the head are staged in LDS, each wave updates its rows and the four partial
-// outputs are summed through LDS.
+// Workgroup = (sequence, head, 64-column slice of Dv), 8 waves; wave w owns 8 columns. A lane is
+// (column c = lane & 7, row group gg = lane >> 3) and keeps the NR rows d = gg * NR .. + NR - 1 of
+// its column's state in registers, so a token costs NR fused updates per lane and three shuffles to
+// sum the eight row groups: no barrier inside the token loop. Tokens are staged 16 at a time:
+// their decays (a = exp(log sigmoid(z) / tau), f32), keys, scaled queries and values go to LDS in
+// one pass (rows past D are zero, so the row loop needs no bound), the outputs of the 16 tokens
+// leave through LDS in another.
 template <typename T, int NR>
-__global__ __launch_bounds__(256) void gla_scan_kernel(const T* __restrict__ q, long q_ld, const T* __restrict__ k,
+__global__ __launch_bounds__(512) void gla_scan_kernel(const T* __restrict__ q, long q_ld, const T* __restrict__ k,
                                                        long k_ld, const T* __restrict__ v, long v_ld,
                                                        const T* __restrict__ z, long z_ld, float* __restrict__ state,
                                                        const int* __restrict__ state_slots,
                                                        const int* __restrict__ row_cu,
                                                        const int* __restrict__ positions, float inv_tau,
                                                        float q_scale, float* __restrict__ o, int H, int D, int Dv) {
-  __shared__ float sa[256], sk[256], sq[256], part[4][64];
+  constexpr int TB = 16, DP = 8 * NR, NT = 512;
+  __shared__ __attribute__((aligned(16))) float sa[TB * DP], sk[TB * DP], sq[TB * DP];
+  __shared__ float sv[TB][64], so[TB][64];
   const int s = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * 64;
   const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int col = c0 + lane;
+  const int cl = 8 * w + (lane & 7), gg = lane >> 3;
+  const int col = c0 + cl;
   const bool live = col < Dv;
   const int r0 = row_cu[s], r1 = row_cu[s + 1];
   const int slot = state_slots[s];
   if (r1 <= r0) return;
   if (slot < 0) {      // padding sequence of a fixed-shape step: defined output, no state
-    if (w == 0 && live)
-      for (int t = r0; t < r1; ++t) o[((long)t * H + h) * Dv + col] = 0.f;
+    for (int i = threadIdx.x; i < (r1 - r0) * 64; i += NT)
+      if (c0 + (i & 63) < Dv) o[((long)(r0 + (i >> 6)) * H + h) * Dv + c0 + (i & 63)] = 0.f;
     return;
   }
   float* S = state + ((long)slot * H + h) * D * Dv;
@@ -291,54 +297,70 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(const T* __restrict__ q, 
   const bool fresh = positions[r0] == 0;
 #pragma unroll
   for (int i = 0; i < NR; ++i) {
-    const int d = w + 4 * i;
+    const int d = gg * NR + i;
     st[i] = (!fresh && live && d < D) ? S[(long)d * Dv + col] : 0.f;
   }
-  // the next token's operands are loaded while the current one is folded into the state
-  const bool stager = (int)threadIdx.x < D;
-  const int d0 = threadIdx.x;
-  float nz = 0.f, nk = 0.f, nq = 0.f, nv = 0.f;
-  if (stager) {
-    nz = (float)z[(long)r0 * z_ld + (long)h * D + d0];
-    nk = (float)k[(long)r0 * k_ld + (long)h * D + d0];
-    nq = (float)q[(long)r0 * q_ld + (long)h * D + d0];
-  }
-  if (live) nv = (float)v[(long)r0 * v_ld + (long)h * Dv + col];
-  for (int t = r0; t < r1; ++t) {
-    const float zz = nz, kk = nk, qq = nq, vv = nv;
-    if (t + 1 < r1) {
-      if (stager) {
-        nz = (float)z[(long)(t + 1) * z_ld + (long)h * D + d0];
-        nk = (float)k[(long)(t + 1) * k_ld + (long)h * D + d0];
-        nq = (float)q[(long)(t + 1) * q_ld + (long)h * D + d0];
-      }
-      if (live) nv = (float)v[(long)(t + 1) * v_ld + (long)h * Dv + col];
-    }
-    if (stager) {
-      // log sigmoid(z) = -softplus(-z), stable on both sides
-      const float ls = zz < 0.f ? zz - log1pf(expf(zz)) : -log1pf(expf(-zz));
-      sa[d0] = expf(ls * inv_tau);
-      sk[d0] = kk;
-      sq[d0] = qq * q_scale;
-    }
-    __syncthreads();
-    float po = 0.f;
-#pragma unroll
-    for (int i = 0; i < NR; ++i) {
-      const int d = w + 4 * i;
+  for (int t0 = r0; t0 < r1; t0 += TB) {
+    const int nb = min(TB, r1 - t0);
+    for (int i = threadIdx.x; i < nb * DP; i += NT) {
+      const int tt = i / DP, d = i - tt * DP;
+      float a = 0.f, kk = 0.f, qq = 0.f;
       if (d < D) {
-        st[i] = fmaf(sa[d], st[i], sk[d] * vv);
-        po = fmaf(sq[d], st[i], po);
+        const long t = t0 + tt;
+        const float zz = (float)z[t * z_ld + (long)h * D + d];
+        // log sigmoid(z) = -softplus(-z), stable on both sides
+        float ls;
+        if constexpr (sizeof(T) == 2) {   // bf16 inputs: hardware exp / log (f32, ~1 ulp)
+          ls = zz < 0.f ? zz - __logf(1.f + __expf(zz)) : -__logf(1.f + __expf(-zz));
+          a = __expf(ls * inv_tau);
+        } else {
+          ls = zz < 0.f ? zz - log1pf(expf(zz)) : -log1pf(expf(-zz));
+          a = expf(ls * inv_tau);
+        }
+        kk = (float)k[t * k_ld + (long)h * D + d];
+        qq = (float)q[t * q_ld + (long)h * D + d] * q_scale;
       }
+      sa[i] = a;
+      sk[i] = kk;
+      sq[i] = qq;
     }
-    part[w][lane] = po;
+    for (int i = threadIdx.x; i < nb * 64; i += NT) {
+      const int tt = i >> 6, c = i & 63;
+      sv[tt][c] = (c0 + c < Dv) ? (float)v[(long)(t0 + tt) * v_ld + (long)h * Dv + c0 + c] : 0.f;
+    }
     __syncthreads();
-    if (w == 0 && live) o[((long)t * H + h) * Dv + col] = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+    for (int tt = 0; tt < nb; ++tt) {
+      const float vv = sv[tt][cl];
+      const f32x4* pa = reinterpret_cast<const f32x4*>(sa + tt * DP + gg * NR);
+      const f32x4* pk = reinterpret_cast<const f32x4*>(sk + tt * DP + gg * NR);
+      const f32x4* pq = reinterpret_cast<const f32x4*>(sq + tt * DP + gg * NR);
+      float po = 0.f;
+#pragma unroll
+      for (int i4 = 0; i4 < NR / 4; ++i4) {
+        const f32x4 a4 = pa[i4], k4 = pk[i4], q4 = pq[i4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          st[4 * i4 + j] = fmaf(a4[j], st[4 * i4 + j], k4[j] * vv);
+          po = fmaf(q4[j], st[4 * i4 + j], po);
+        }
+      }
+      po += __shfl_xor(po, 8, 64);
+      po += __shfl_xor(po, 16, 64);
+      po += __shfl_xor(po, 32, 64);
+      if (gg == 0) so[tt][cl] = po;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nb * 64; i += NT) {
+      const int tt = i >> 6, c = i & 63;
+      if (c0 + c < Dv) o[((long)(t0 + tt) * H + h) * Dv + c0 + c] = so[tt][c];
+    }
+    // (the next block's staging overwrites sa / sk / sq / sv, which every wave finished reading
+    // at the barrier above; so is rewritten only after the next block's first barrier)
   }
   if (live) {
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
-      const int d = w + 4 * i;
+      const int d = gg * NR + i;
       if (d < D) S[(long)d * Dv + col] = st[i];
     }
   }
@@ -448,12 +470,12 @@ static int gla_scan_t(const T* q, long q_ld, const T* k, long k_ld, const T* v, 
   dim3 grid(nseq, H, (Dv + 63) / 64);
   const float it = 1.f / tau;
 #define BFLY_GLA(NR)                                                                                              \
-  gla_scan_kernel<T, NR><<<grid, 256, 0, s>>>(q, q_ld, k, k_ld, v, v_ld, z, z_ld, state, state_slots, row_cu, positions, \
+  gla_scan_kernel<T, NR><<<grid, 512, 0, s>>>(q, q_ld, k, k_ld, v, v_ld, z, z_ld, state, state_slots, row_cu, positions, \
                                               it, q_scale, o, H, D, Dv)
-  if (D <= 32) BFLY_GLA(8);
-  else if (D <= 64) BFLY_GLA(16);
-  else if (D <= 128) BFLY_GLA(32);
-  else if (D <= 256) BFLY_GLA(64);
+  if (D <= 32) BFLY_GLA(4);
+  else if (D <= 64) BFLY_GLA(8);
+  else if (D <= 128) BFLY_GLA(16);
+  else if (D <= 256) BFLY_GLA(32);
   else return -1;
 #undef BFLY_GLA
   return 0;
