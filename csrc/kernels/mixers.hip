@@ -187,20 +187,39 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
   for (int t = 0; t < DVT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int kp = (min(keep_first, pmax + 1) + BS - 1) / BS;          // pages of the kept prefix
   const int wp0 = max(max(0, pmin - window + 1) / BS, kp), wp1 = pmax / BS;
-  for (int pg = 0; pg <= wp1; pg = (pg + 1 == kp && wp0 > kp) ? wp0 : pg + 1) {
-    if (pg >= kp && pg < wp0) { pg = wp0 - 1; continue; }
-    const long blk = (long)tab[pg] * G + g;
-    const bf16* Kp = k_cache + blk * BS * D;
-    const bf16* Vp = v_cache + blk * Dv * BS;
+  // pages: the kept prefix [0, kp), then the window [wp0, wp1]; the next page's K fragments are
+  // loaded before the current page is multiplied, and a page's V fragments before its scores
+  auto next_page = [&](int pg) { return pg + 1 < kp ? pg + 1 : max(pg + 1, wp0); };
+  auto load_k = [&](int pg, bf16x8 (&kf)[2][DS]) {
+    const bf16* Kp = k_cache + ((long)tab[pg] * G + g) * BS * D;
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+      for (int ds = 0; ds < DS; ++ds)
+        kf[kh][ds] = *reinterpret_cast<const bf16x8*>(Kp + (long)(16 * kh + qr) * D + 32 * ds + 8 * gg);
+  };
+  int pg = kp > 0 ? 0 : wp0;
+  bf16x8 kf[2][DS];
+  if (pg <= wp1) load_k(pg, kf);
+  while (pg <= wp1) {
+    const int npg = next_page(pg);
+    const bf16* Vp = v_cache + ((long)tab[pg] * G + g) * Dv * BS;
+    bf16x8 vf[DVT];
+#pragma unroll
+    for (int t = 0; t < DVT; ++t) {
+      const bf16* vr = Vp + (long)(16 * t + qr) * BS + 4 * gg;
+      const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vr);
+      const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vr + 16);
+      vf[t] = bf16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+    }
+    bf16x8 nkf[2][DS];
+    if (npg <= wp1) load_k(npg, nkf);
     f32x4 st[2];
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh) {
       st[kh] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ds = 0; ds < DS; ++ds) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Kp + (long)(16 * kh + qr) * D + 32 * ds + 8 * gg);
-        st[kh] = mfma16(kf, qf[ds], st[kh]);
-      }
+      for (int ds = 0; ds < DS; ++ds) st[kh] = mfma16(kf[kh][ds], qf[ds], st[kh]);
     }
     float sc[8], mx = -INFINITY;
 #pragma unroll
@@ -230,14 +249,17 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
     m = mn;
 #pragma unroll
     for (int t = 0; t < DVT; ++t) {
-      const bf16* vr = Vp + (long)(16 * t + qr) * BS + 4 * gg;
-      const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vr);
-      const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vr + 16);
-      const bf16x8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[t][i] *= corr;
-      o[t] = mfma16(vf, pb, o[t]);
+      o[t] = mfma16(vf[t], pb, o[t]);
     }
+    if (npg <= wp1) {
+#pragma unroll
+      for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) kf[kh][ds] = nkf[kh][ds];
+    }
+    pg = npg;
   }
   if (!rv) return;
   const float inv = 1.f / l;
