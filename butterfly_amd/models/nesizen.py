@@ -325,17 +325,27 @@ class NesizenLM:
         p, eps = self.p, self.cfg.norm_eps
         meta = self._step_meta(fb)
         xs = ops.embed_norm_streams(fb.input_ids, p["embed"], p["embed.norm"], eps, NORM_OFFSET, self.streams)
-        for sp in self.specs:
+        # sublayers in order; each stream update is fused with the next sublayer's mixed-in norm
+        subs = [(sp, q) for sp in self.specs for q in ((1, 2) if sp["ffn"] else (1,))]
+        sp0 = subs[0][0]
+        h = ops.hc_pre(xs, p[f"l{sp0['index']}.hc1.in"], p[f"l{sp0['index']}.norm1"], eps, NORM_OFFSET, self.dtype)
+        for n, (sp, q) in enumerate(subs):
             pre = f"l{sp['index']}."
-            h = ops.hc_pre(xs, p[pre + "hc1.in"], p[pre + "norm1"], eps, NORM_OFFSET, self.dtype)
-            y = self._attention(sp, pre, h, fb, meta, kv_caches) if sp["type"] == "attention" else \
-                self._gla(sp, pre, h, fb, meta)
-            ops.hc_post_(xs, y, p[pre + "hc1.mix"], p[pre + "hc1.out"])
-            if sp["ffn"]:
-                h = ops.hc_pre(xs, p[pre + "hc2.in"], p[pre + "norm2"], eps, NORM_OFFSET, self.dtype)
+            if q == 2:
                 y = self._ffn(sp["ffn"], pre, h)
-                ops.hc_post_(xs, y, p[pre + "hc2.mix"], p[pre + "hc2.out"])
-            if self.layer_probe is not None:
+            elif sp["type"] == "attention":
+                y = self._attention(sp, pre, h, fb, meta, kv_caches)
+            else:
+                y = self._gla(sp, pre, h, fb, meta)
+            hc = pre + f"hc{q}."
+            if n + 1 < len(subs):
+                nsp, nq = subs[n + 1]
+                npre = f"l{nsp['index']}."
+                h = ops.hc_post_pre_(xs, y, p[hc + "mix"], p[hc + "out"], p[npre + f"hc{nq}.in"], p[npre + f"norm{nq}"],
+                                     eps, NORM_OFFSET, self.dtype)
+            else:
+                ops.hc_post_(xs, y, p[hc + "mix"], p[hc + "out"])
+            if self.layer_probe is not None and (q == 2 or not sp["ffn"]):
                 self.layer_probe(sp["index"], xs.sum(1))
         x = ops.hc_final(xs, p["final.norm"], eps, NORM_OFFSET, fb.logits_idx, self.dtype)
         return ops.linear_act(x, p["head"])

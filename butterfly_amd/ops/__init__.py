@@ -781,6 +781,17 @@ def hc_post_(xs, y, mix, w_out):
     return xs
 
 
+def hc_post_pre_(xs, y, mix, w_out, w_in2, norm_w2, eps: float, offset: float, out_dtype):
+    """hc_post_ followed by the next sublayer's hc_pre on the updated streams, in one kernel (the
+    residual update fused with the following norm, as the other families' add + norm)."""
+    if not _gpu(xs):
+        ref.hc_post_(xs, y, mix, w_out)
+        return ref.hc_pre(xs, w_in2, norm_w2, eps, offset, out_dtype)
+    out = _empty(xs.shape[0], xs.shape[2], dtype=out_dtype, device=xs.device)
+    torch.ops.bfly.hc_post_pre(xs, y, mix, w_out, w_in2, norm_w2, eps, offset, out)
+    return out
+
+
 def hc_final(xs, norm_w, eps: float, offset: float, idx, out_dtype):
     """Sum of the streams of rows `idx` (None: all), RMS-normed with weight (w + offset)."""
     if not _gpu(xs):

@@ -84,6 +84,20 @@ void hc_post(Tensor& xs, const Tensor& y, const Tensor& mix, const Tensor& w_out
                        (int)S, (int)W, is_f32(y), cur_stream());
 }
 
+void hc_post_pre(Tensor& xs, const Tensor& y, const Tensor& mix, const Tensor& w_out, const Tensor& w_in2,
+                 const Tensor& norm_w2, double eps, double offset, Tensor& out) {
+  CHK_GPU(xs); CHK_F32(xs); CHK_F32(mix); CHK_F32(w_out); CHK_F32(w_in2); CHK_F32(norm_w2); CHK_SAME(y, out);
+  TORCH_CHECK(xs.dim() == 3 && y.dim() == 2 && y.is_contiguous() && out.dim() == 2 && out.is_contiguous(),
+              "hc_post_pre: layouts");
+  const int64_t T = xs.size(0), S = xs.size(1), W = xs.size(2);
+  TORCH_CHECK(S <= 16, "hc_post_pre: at most 16 residual streams");
+  TORCH_CHECK(mix.numel() == S * S && w_out.numel() == S && w_in2.numel() == S && norm_w2.numel() == W &&
+                  y.size(0) == T && y.size(1) == W && out.size(0) == T && out.size(1) == W, "hc_post_pre: shapes");
+  bfly::launch_hc_post_pre(xs.data_ptr<float>(), y.data_ptr(), mix.data_ptr<float>(), w_out.data_ptr<float>(),
+                           w_in2.data_ptr<float>(), norm_w2.data_ptr<float>(), (float)eps, (float)offset, out.data_ptr(),
+                           (int)T, (int)S, (int)W, is_f32(y), cur_stream());
+}
+
 void hc_final(const Tensor& xs, const Tensor& norm_w, double eps, double offset, const optional<Tensor>& idx,
               Tensor& out) {
   CHK_GPU(xs); CHK_F32(xs); CHK_F32(norm_w);
@@ -266,6 +280,8 @@ TORCH_LIBRARY_FRAGMENT(bfly, m) {
   m.def("embed_norm_streams(Tensor ids, Tensor table, Tensor norm_w, float eps, float offset, Tensor(a!) xs) -> ()");
   m.def("hc_pre(Tensor xs, Tensor w_in, Tensor norm_w, float eps, float offset, Tensor(a!) out) -> ()");
   m.def("hc_post(Tensor(a!) xs, Tensor y, Tensor mix, Tensor w_out) -> ()");
+  m.def("hc_post_pre(Tensor(a!) xs, Tensor y, Tensor mix, Tensor w_out, Tensor w_in2, Tensor norm_w2, float eps, "
+        "float offset, Tensor(b!) out) -> ()");
   m.def("hc_final(Tensor xs, Tensor norm_w, float eps, float offset, Tensor? idx, Tensor(a!) out) -> ()");
   m.def("rope_partial_kv(Tensor(a!) q, Tensor(b!)? k, Tensor? v, Tensor positions, Tensor inv_freq, Tensor? slots, "
         "Tensor(c!)? k_cache, Tensor(d!)? v_cache) -> ()");
@@ -288,6 +304,7 @@ TORCH_LIBRARY_IMPL(bfly, CUDA, m) {
   m.impl("embed_norm_streams", &embed_norm_streams);
   m.impl("hc_pre", &hc_pre);
   m.impl("hc_post", &hc_post);
+  m.impl("hc_post_pre", &hc_post_pre);
   m.impl("hc_final", &hc_final);
   m.impl("rope_partial_kv", &rope_partial_kv);
   m.impl("row_seq", &row_seq);

@@ -28,6 +28,10 @@ void launch_hc_pre(const float* xs, const float* w_in, const float* norm_w, floa
 // xs[t, r] <- sum_s mix[s, r] xs[t, s] + w_out[r] y[t]   (all streams at once from the old ones)
 void launch_hc_post(float* xs, const void* y, const float* mix, const float* w_out, int T, int S, int W, bool f32,
                     hipStream_t s);
+// launch_hc_post, then launch_hc_pre of the next sublayer (w_in2, norm_w2) on the updated streams
+void launch_hc_post_pre(float* xs, const void* y, const float* mix, const float* w_out, const float* w_in2,
+                        const float* norm_w2, float eps, float offset, void* out, int T, int S, int W, bool f32,
+                        hipStream_t s);
 // out[i] = rms(sum_s xs[idx[i], s]) * (w + offset); idx == nullptr: every row
 void launch_hc_final(const float* xs, const float* norm_w, float eps, float offset, const long* idx, void* out,
                      int R, int S, int W, bool f32, hipStream_t s);

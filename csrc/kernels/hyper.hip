@@ -76,6 +76,42 @@ __global__ __launch_bounds__(256) void hc_post_kernel(float* __restrict__ xs, co
   }
 }
 
+// hc_post followed by the next sublayer's hc_pre on the updated streams, one pass over the row's
+// streams for both (the same thread owns a column in both halves, so it rereads what it wrote).
+template <typename T>
+__global__ __launch_bounds__(256) void hc_post_pre_kernel(float* __restrict__ xs, const T* __restrict__ y,
+                                                          const float* __restrict__ mix,
+                                                          const float* __restrict__ w_out,
+                                                          const float* __restrict__ w_in2,
+                                                          const float* __restrict__ norm_w2, float eps, float offset,
+                                                          T* __restrict__ out, int S, int W) {
+  __shared__ float red[16];
+  const long t = blockIdx.x;
+  float* x = xs + t * S * W;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float old[kMaxStreams];
+    for (int s = 0; s < S; ++s) old[s] = x[(long)s * W + c];
+    const float yv = (float)y[t * W + c];
+    float u = 0.f;
+    for (int r = 0; r < S; ++r) {
+      float v = 0.f;
+      for (int s = 0; s < S; ++s) v = fmaf(mix[s * S + r], old[s], v);
+      v = fmaf(w_out[r], yv, v);
+      x[(long)r * W + c] = v;
+      u = fmaf(w_in2[r], v, u);
+    }
+    ss = fmaf(u, u, ss);
+  }
+  ss = block_sum(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float u = 0.f;
+    for (int s = 0; s < S; ++s) u = fmaf(w_in2[s], x[(long)s * W + c], u);
+    out[t * W + c] = (T)(u * r * (norm_w2[c] + offset));
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void hc_final_kernel(const float* __restrict__ xs, const float* __restrict__ norm_w,
                                                        float eps, float offset, const long* __restrict__ idx,
@@ -120,6 +156,16 @@ void launch_hc_post(float* xs, const void* y, const float* mix, const float* w_o
   if (T <= 0) return;
   if (f32) hc_post_kernel<float><<<T, 256, 0, s>>>(xs, (const float*)y, mix, w_out, S, W);
   else hc_post_kernel<bf16><<<T, 256, 0, s>>>(xs, (const bf16*)y, mix, w_out, S, W);
+}
+
+void launch_hc_post_pre(float* xs, const void* y, const float* mix, const float* w_out, const float* w_in2,
+                        const float* norm_w2, float eps, float offset, void* out, int T, int S, int W, bool f32,
+                        hipStream_t s) {
+  if (T <= 0) return;
+  if (f32)
+    hc_post_pre_kernel<float><<<T, 256, 0, s>>>(xs, (const float*)y, mix, w_out, w_in2, norm_w2, eps, offset, (float*)out, S, W);
+  else
+    hc_post_pre_kernel<bf16><<<T, 256, 0, s>>>(xs, (const bf16*)y, mix, w_out, w_in2, norm_w2, eps, offset, (bf16*)out, S, W);
 }
 
 void launch_hc_final(const float* xs, const float* norm_w, float eps, float offset, const long* idx, void* out,

@@ -111,8 +111,14 @@ def test_streams_and_offset_norm(target, S):
     want_h = O.norm_zero_centered(O.streams_read(xs64, w_in), nw, eps)
     assert (h.cpu().to(F64) - want_h).abs().max() < (1e-4 if dt == torch.float32 else 3e-2)
     y = bf(torch.randn(T, W, generator=g, dtype=F64))
-    ops.hc_post_(xs, y.to(dev, dt), f32(mix), f32(w_out))
     want_xs = O.streams_write(xs64, y, mix, w_out)
+    # the fused form: stream update, then the next sublayer's mixed-in norm of the new streams
+    xs2, w_in2, nw2 = xs.clone(), bf(torch.randn(S, generator=g, dtype=F64)), bf(0.3 * torch.randn(W, generator=g, dtype=F64))
+    h2 = ops.hc_post_pre_(xs2, y.to(dev, dt), f32(mix), f32(w_out), f32(w_in2), f32(nw2), eps, 1.0, dt)
+    want_h2 = O.norm_zero_centered(O.streams_read(want_xs, w_in2), nw2, eps)
+    assert (xs2.cpu().to(F64).permute(1, 0, 2) - want_xs).abs().max() < 1e-3
+    assert (h2.cpu().to(F64) - want_h2).abs().max() < (1e-4 if dt == torch.float32 else 3e-2)
+    ops.hc_post_(xs, y.to(dev, dt), f32(mix), f32(w_out))
     assert (xs.cpu().to(F64).permute(1, 0, 2) - want_xs).abs().max() < 1e-3
     idx = torch.tensor([T - 1, 0, 4])
     fin = ops.hc_final(xs, f32(nw), eps, 1.0, idx.to(dev), dt)
