@@ -1,7 +1,9 @@
 // Shape-generic GEMM family: any (M, N, K), bf16 or f32 operands, f32 accumulation in K order
 // (the sum of an output element never depends on M or on the other rows of the batch).
-// 64 x 64 output tile, 16-deep K step, 256 threads with a 4 x 4 register block each; operands
-// are staged through LDS as f32 with bounds checks, so no shape or alignment restriction.
+// 64 x 64 output tile and 256 threads in both forms, operands staged through LDS with bounds
+// checks, so no shape or alignment restriction. f32 operands: 16-deep K step, a 4 x 4 register
+// block per thread on the VALU. bf16 operands: 64-deep K step staged as bf16, a 32 x 32 quadrant
+// per wave as 2 x 2 MFMA 16x16x32 tiles (tile_mac_mfma below).
 // The same tile core serves the plain projection (bias / squared-ReLU epilogues) and the two
 // grouped expert GEMMs of a score-routed MoE with clamped GLU experts: rows are grouped by
 // expert (moe_sort_kernel), the up kernel gathers token rows scaled by their routing score and
