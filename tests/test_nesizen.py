@@ -166,7 +166,10 @@ def _paged(k, v, bs, perm_seed, dev, dt, extra=3):
 
 
 @pytest.mark.parametrize("window,keep,H,G,D,Dv", [(9, 3, 4, 2, 16, 8), (33, 0, 2, 2, 8, 72), (40, 35, 3, 1, 24, 16),
-                                                  (1, 2, 2, 1, 8, 8), (500, 0, 2, 2, 8, 8)])
+                                                  (1, 2, 2, 1, 8, 8), (500, 0, 2, 2, 8, 8),
+                                                  # head sizes the MFMA form of the bf16 kernel takes
+                                                  (9, 3, 4, 2, 64, 64), (33, 34, 2, 1, 32, 128), (64, 0, 6, 3, 128, 32),
+                                                  (31, 1, 2, 2, 256, 256), (500, 70, 4, 1, 64, 32)])
 def test_attention_window_edges(target, window, keep, H, G, D, Dv):
     """A query aimed at one key (scaled so that its score stands out) sees it just inside the
     window, not just outside; among the kept first positions, not at the next one; across page
@@ -319,6 +322,18 @@ def cfg_c():
     ], width=48, vocab=50, streams=4, eps=1e-6)
 
 
+def cfg_d():
+    """Head sizes and widths that the MFMA kernels tile (bf16): attention 64 / 32 with a window of
+    40 and 6 kept tokens read again by a later layer with a longer window, GLA 64 / 64 and
+    32 / 128, two of eight experts."""
+    return O.config([
+        O.gla_layer(2, 64, 64, 16.0, O.dense(256)),
+        O.attn_layer(4, 2, 64, 32, 32, 1e6, 0.125, 40, 6, O.moe(8, 2, 64, 1.0)),
+        O.gla_layer(1, 32, 128, 4.0, None),
+        O.attn_layer(4, 2, 64, 32, 32, 1e6, 0.125, 70, 0, O.moe(8, 2, 64, 1.0), kv_from=1),
+    ], width=128, vocab=256, streams=3, eps=1e-6)
+
+
 _ORACLE = {}
 
 
@@ -369,7 +384,7 @@ def replay(eng, reqs, schedule):
     return {n: torch.cat(v) for n, v in out.items()}
 
 
-@pytest.mark.parametrize("name,mk", [("a", cfg_a), ("b", cfg_b), ("c", cfg_c)])
+@pytest.mark.parametrize("name,mk", [("a", cfg_a), ("b", cfg_b), ("c", cfg_c), ("d", cfg_d)])
 def test_prompt_decode_and_portions(target, tmp_path, name, mk):
     """One request: whole prompt; prompt then token-by-token decoding (long); portions of many
     sizes down to two tokens, ending on single tokens. Same logits as the oracle every way."""
@@ -391,7 +406,7 @@ def test_prompt_decode_and_portions(target, tmp_path, name, mk):
     assert_rows(got, want[:3], dt, "first tokens")
 
 
-@pytest.mark.parametrize("name,mk", [("a", cfg_a), ("c", cfg_c)])
+@pytest.mark.parametrize("name,mk", [("a", cfg_a), ("c", cfg_c), ("d", cfg_d)])
 def test_mixed_batches_reuse_pages_and_slots(target, tmp_path, name, mk):
     """Six requests of unequal length through three state slots and a cache that holds about
     half of them: portions beside decoded tokens of other requests, requests that pause,
