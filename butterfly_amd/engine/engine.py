@@ -123,6 +123,8 @@ class LLMEngine:
         # kernels have an f32 form; the bf16-only families refuse it on the GPU)
         want32 = str(engine_cfg.dtype).lower() in ("fp32", "float32", "f32")
         dtype = torch.float32 if (self.device.type != "cuda" or want32) else torch.bfloat16
+        if want32 and self.device.type == "cuda" and model is None and cfg.arch != "nesizen":
+            raise NotImplementedError(f"{cfg.arch} GPU kernels are bf16 only (EngineConfig.dtype = 'bf16')")
         self.model = model or build_model(cfg, shard, device=self.device, dtype=dtype, comm=self.comm)
         if model is None:
             self.model.init_random(engine_cfg.seed)

@@ -93,8 +93,6 @@ class TransformerLM:
         self.rowscale_rows = (flags.get("BFLY_NORM_ROWSCALE_MAX_ROWS")
                               if (self.device.type == "cuda" and cfg.norm == "rms" and self.tp == 1
                                   and not cfg.is_moe and flags.get("BFLY_NORM_ROWSCALE")) else 0)
-        if self.device.type == "cuda" and dtype != torch.bfloat16:
-            raise NotImplementedError(f"{cfg.arch} GPU kernels are bf16 only (EngineConfig.dtype = 'bf16')")
         if self.device.type == "cuda" and cfg.head_dim != 128:
             raise NotImplementedError(f"GPU attention kernels need head_dim 128 (got {cfg.head_dim})")
         self.p: dict[str, torch.Tensor] = {}
