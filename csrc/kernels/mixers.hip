@@ -136,14 +136,17 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
   }
 }
 
-// MFMA form for bf16 with 32-token pages, D = 32 DS, Dv = 16 DVT: one wave per 16 consecutive
-// rows of a sequence and one query head, no LDS. Per page: S^T = K Q^T (16x16x32 tiles, K rows
-// read as 16-byte segments straight from the page), masks and an online softmax in f32 (the four
-// lanes that share a query row combine by shuffles), then O^T += V^T P with the page's keys as
-// the MFMA k index in the order the score tiles leave them (keys 4g..4g+3 and 16+4g..16+4g+3 in
-// lane group g), which the transposed V page serves with two 8-byte reads. The softmax is
-// seeded with the sink (m = sink, l = 1). Pages outside the window and the kept prefix are
-// skipped; the per-element mask settles the edges.
+// MFMA form for bf16 with 32-token pages, D = 32 DS, Dv = 16 DVT. A workgroup of 4 waves owns 16
+// consecutive rows of a sequence and one query head; the visible pages (the kept prefix, then the
+// window) are dealt round-robin to the waves, each wave keeps its own online softmax, and wave 0
+// folds the other three in through LDS at the end (a decoded row's ~window / 32 pages are thus
+// walked by four waves, a prompt tile's by four as well). Per page, no LDS: S^T = K Q^T
+// (16x16x32 tiles, K rows read as 16-byte segments straight from the page), masks and softmax
+// in f32 (the four lanes that share a query row combine by shuffles), then O^T += V^T P with the
+// page's keys as the MFMA k index in the order the score tiles leave them (keys 4g..4g+3 and
+// 16+4g..16+4g+3 in lane group g), which the transposed V page serves with two 8-byte reads.
+// The next page's K and V fragments are loaded before the current page is multiplied. The sink
+// seeds wave 0's softmax (m = sink, l = 1). The per-element mask settles the window edges.
 template <int DS, int DVT>
 __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __restrict__ q, long q_ld,
                                                                const bf16* __restrict__ k_cache,
@@ -155,8 +158,12 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
                                                                const float* __restrict__ sink,
                                                                bf16* __restrict__ out, int H, int G) {
   constexpr int D = 32 * DS, Dv = 16 * DVT, BS = 32;
-  const int lane = threadIdx.x & 63;
-  int tile = blockIdx.x * 4 + (threadIdx.x >> 6);
+  extern __shared__ float smem[];          // o of waves 1-3 [3][DVT][4][64] | m [3][16] | l [3][16]
+  float* so = smem;
+  float* sm = smem + 3 * DVT * 256;
+  float* sl = sm + 48;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int tile = blockIdx.x;
   const int h = blockIdx.y, g = h / (H / G);
   int s = 0, row0 = 0, rend = 0;
   for (; s < nseq; ++s) {
@@ -165,7 +172,7 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
     if (tile < nt) { row0 = a + 16 * tile; rend = b; break; }
     tile -= nt;
   }
-  if (s >= nseq) return;
+  if (s >= nseq) return;                   // (the whole workgroup: the tile is per workgroup)
   const int qr = lane & 15, gg = lane >> 4;
   const bool rv = row0 + qr < rend;
   const long row = rv ? row0 + qr : row0;
@@ -181,30 +188,23 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
   for (int ds = 0; ds < DS; ++ds)
     qf[ds] = *reinterpret_cast<const bf16x8*>(q + row * q_ld + (long)h * D + 32 * ds + 8 * gg);
   const int* tab = tables + (long)s * max_blocks;
-  float m = sink[h], l = 1.f;
+  float m = wave == 0 ? sink[h] : -1e30f, l = wave == 0 ? 1.f : 0.f;
   f32x4 o[DVT];
 #pragma unroll
   for (int t = 0; t < DVT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int kp = (min(keep_first, pmax + 1) + BS - 1) / BS;          // pages of the kept prefix
   const int wp0 = max(max(0, pmin - window + 1) / BS, kp), wp1 = pmax / BS;
-  // pages: the kept prefix [0, kp), then the window [wp0, wp1]; the next page's K fragments are
-  // loaded before the current page is multiplied, and a page's V fragments before its scores
-  auto next_page = [&](int pg) { return pg + 1 < kp ? pg + 1 : max(pg + 1, wp0); };
-  auto load_k = [&](int pg, bf16x8 (&kf)[2][DS]) {
-    const bf16* Kp = k_cache + ((long)tab[pg] * G + g) * BS * D;
+  const int npages = kp + max(0, wp1 - wp0 + 1);
+  auto page_of = [&](int i) { return i < kp ? i : wp0 + (i - kp); };
+  auto load_kv = [&](int pg, bf16x8 (&kf)[2][DS], bf16x8 (&vf)[DVT]) {
+    const long blk = (long)tab[pg] * G + g;
+    const bf16* Kp = k_cache + blk * BS * D;
+    const bf16* Vp = v_cache + blk * Dv * BS;
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh)
 #pragma unroll
       for (int ds = 0; ds < DS; ++ds)
         kf[kh][ds] = *reinterpret_cast<const bf16x8*>(Kp + (long)(16 * kh + qr) * D + 32 * ds + 8 * gg);
-  };
-  int pg = kp > 0 ? 0 : wp0;
-  bf16x8 kf[2][DS];
-  if (pg <= wp1) load_k(pg, kf);
-  while (pg <= wp1) {
-    const int npg = next_page(pg);
-    const bf16* Vp = v_cache + ((long)tab[pg] * G + g) * Dv * BS;
-    bf16x8 vf[DVT];
 #pragma unroll
     for (int t = 0; t < DVT; ++t) {
       const bf16* vr = Vp + (long)(16 * t + qr) * BS + 4 * gg;
@@ -212,8 +212,15 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
       const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vr + 16);
       vf[t] = bf16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
     }
-    bf16x8 nkf[2][DS];
-    if (npg <= wp1) load_k(npg, nkf);
+  };
+  bf16x8 kf[2][DS], vf[DVT];
+  int pi = wave;
+  if (pi < npages) load_kv(page_of(pi), kf, vf);
+  while (pi < npages) {
+    const int pg = page_of(pi);
+    const int ni = pi + 4;
+    bf16x8 nkf[2][DS], nvf[DVT];
+    if (ni < npages) load_kv(page_of(ni), nkf, nvf);
     f32x4 st[2];
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh) {
@@ -253,13 +260,41 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
       for (int i = 0; i < 4; ++i) o[t][i] *= corr;
       o[t] = mfma16(vf[t], pb, o[t]);
     }
-    if (npg <= wp1) {
+    if (ni < npages) {
 #pragma unroll
       for (int kh = 0; kh < 2; ++kh)
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) kf[kh][ds] = nkf[kh][ds];
+#pragma unroll
+      for (int t = 0; t < DVT; ++t) vf[t] = nvf[t];
     }
-    pg = npg;
+    pi = ni;
+  }
+  if (wave > 0) {
+    float* po = so + (long)(wave - 1) * DVT * 256;
+#pragma unroll
+    for (int t = 0; t < DVT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) po[(t * 4 + i) * 64 + lane] = o[t][i];
+    if (gg == 0) {
+      sm[(wave - 1) * 16 + qr] = m;
+      sl[(wave - 1) * 16 + qr] = l;
+    }
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int u = 0; u < 3; ++u) {
+    const float mu = sm[u * 16 + qr], lu = sl[u * 16 + qr];
+    const float mn = fmaxf(m, mu);
+    const float c0 = __expf(m - mn), cu = __expf(mu - mn);
+    l = l * c0 + lu * cu;
+    m = mn;
+    const float* po = so + (long)u * DVT * 256;
+#pragma unroll
+    for (int t = 0; t < DVT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[t][i] = o[t][i] * c0 + po[(t * 4 + i) * 64 + lane] * cu;
   }
   if (!rv) return;
   const float inv = 1.f / l;
@@ -431,11 +466,11 @@ template <int DS>
 static bool attn_mfma_dv(const bf16* q, long q_ld, const bf16* kc, const bf16* vc, const int* tables, int max_blocks,
                          const int* row_cu, int nseq, const int* positions, float scale, int window, int keep_first,
                          const float* sink, bf16* out, int T, int H, int G, int Dv, hipStream_t s) {
-  // every sequence adds at most one partly filled 16-row tile
-  dim3 grid(((T + 15) / 16 + nseq + 3) / 4, H);
-#define BFLY_ATT(DVT)                                                                                            \
-  attn_window_mfma_kernel<DS, DVT><<<grid, 256, 0, s>>>(q, q_ld, kc, vc, tables, max_blocks, row_cu, nseq, positions, \
-                                                        scale, window, keep_first, sink, out, H, G)
+  // one workgroup per 16-row tile; every sequence adds at most one partly filled tile
+  dim3 grid((T + 15) / 16 + nseq, H);
+#define BFLY_ATT(DVT)                                                                                          \
+  attn_window_mfma_kernel<DS, DVT><<<grid, 256, (3 * DVT * 256 + 96) * sizeof(float), s>>>(                    \
+      q, q_ld, kc, vc, tables, max_blocks, row_cu, nseq, positions, scale, window, keep_first, sink, out, H, G)
   switch (Dv) {
     case 32: BFLY_ATT(2); return true;
     case 64: BFLY_ATT(4); return true;
