@@ -253,12 +253,13 @@ void moe_glu_ffn(const Tensor& x, const Tensor& topk_ids, const Tensor& topk_w, 
   int* ntiles = tiles + 2 * mt;
   hipStream_t s = cur_stream();
   const bool f32 = is_f32(x);
-  bfly::launch_moe_sort(topk_ids.data_ptr<int>(), (int)TK, (int)E, perm, offsets, tiles, ntiles, s);
+  const int tr = bfly::moe_tile_rows((int)TK, (int)E, f32);
+  bfly::launch_moe_sort(topk_ids.data_ptr<int>(), (int)TK, (int)E, perm, offsets, tiles, ntiles, tr, s);
   bfly::launch_moe_glu_up(x.data_ptr(), x.stride(0), topk_w.data_ptr<float>(), (int)K, perm, offsets, tiles, ntiles,
                           (int)mt, gate_up_w.data_ptr(), (float)limit, (float)alpha, hmid.data_ptr(), (int)Hd, (int)F,
-                          f32, s);
+                          f32, tr, s);
   bfly::launch_moe_down(hmid.data_ptr(), perm, offsets, tiles, ntiles, (int)mt, down_w.data_ptr(), y.data_ptr<float>(),
-                        (int)Hd, (int)F, f32, s);
+                        (int)Hd, (int)F, f32, tr, s);
   bfly::launch_moe_sum(y.data_ptr<float>(), (int)K, out.data_ptr(), (int)T, (int)Hd, f32, s);
 }
 

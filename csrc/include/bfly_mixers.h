@@ -72,16 +72,19 @@ void launch_gla_out(const float* o, const void* g, long g_ld, const float* norm_
 void launch_moe_topk_scores(const float* logits, int top_k, int scoring, bool renorm, int* ids, float* w, int T, int E,
                             hipStream_t s);
 // Group the T*K (token, choice) pairs by expert: perm [TK] pair indices grouped by expert,
-// offsets [E + 1], tiles [max_tiles][2] = (expert, first row) of every 64-row tile, ntiles [1].
-void launch_moe_sort(const int* ids, int TK, int E, int* perm, int* offsets, int* tiles, int* ntiles, hipStream_t s);
+// offsets [E + 1], tiles [max_tiles][2] = (expert, first row) of every tile_rows-row tile, ntiles [1].
+void launch_moe_sort(const int* ids, int TK, int E, int* perm, int* offsets, int* tiles, int* ntiles, int tile_rows,
+                     hipStream_t s);
 int moe_sort_max_tiles(int TK, int E);
+// rows per tile of the grouped expert GEMMs for this problem (64, or 128 for large bf16 groups)
+int moe_tile_rows(int TK, int E, bool f32);
 // hmid[r, f] = glu(gate, up) of expert e(r) on (w x) for grouped row r
 void launch_moe_glu_up(const void* x, long ldx, const float* topk_w, int K, const int* perm, const int* offsets,
                        const int* tiles, const int* ntiles, int max_tiles, const void* gate_up_w, float limit,
-                       float alpha, void* hmid, int Hd, int F, bool f32, hipStream_t s);
+                       float alpha, void* hmid, int Hd, int F, bool f32, int tile_rows, hipStream_t s);
 // y[perm[r], :] = down_e(r) hmid[r]     (y f32, pair order)
 void launch_moe_down(const void* hmid, const int* perm, const int* offsets, const int* tiles, const int* ntiles,
-                     int max_tiles, const void* down_w, float* y, int Hd, int F, bool f32, hipStream_t s);
+                     int max_tiles, const void* down_w, float* y, int Hd, int F, bool f32, int tile_rows, hipStream_t s);
 // out[t] = sum_j y[t * K + j]
 void launch_moe_sum(const float* y, int K, void* out, int T, int Hd, bool f32, hipStream_t s);
 

@@ -90,10 +90,12 @@ __global__ void relu2_kernel(T* x, long n) {
 }
 
 // One workgroup. counts -> offsets -> placement (order inside an expert's group is arbitrary:
-// every grouped row is computed on its own and lands at its pair index) -> 64-row tile list.
+// every grouped row is computed on its own and lands at its pair index) -> list of tile_rows-row
+// tiles.
 __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int TKp, int E,
                                                         int* __restrict__ perm, int* __restrict__ offsets,
-                                                        int* __restrict__ tiles, int* __restrict__ ntiles) {
+                                                        int* __restrict__ tiles, int* __restrict__ ntiles,
+                                                        int tile_rows) {
   __shared__ int cnt[1025], cur[1024];
   for (int e = threadIdx.x; e <= E; e += blockDim.x) cnt[e] = 0;
   __syncthreads();
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ 
       const int c = cnt[e];
       offsets[e] = run;
       cur[e] = run;
-      for (int r = 0; r < c; r += 64) {
+      for (int r = 0; r < c; r += tile_rows) {
         tiles[2 * nt] = e;
         tiles[2 * nt + 1] = run + r;
         ++nt;
@@ -299,78 +301,106 @@ __device__ __forceinline__ bf16x8 load_row8(const RowRef r, int k, int K) {
   return v;
 }
 
-// acc[tn][tm][i] += sum_k X(m, k) W(n, k) with m = 32 * (wave >> 1) + 16 tm + (lane & 15) and
-// n = 32 * (wave & 1) + 16 tn + 4 * (lane >> 4) + i inside the tile; rowX(r) / rowW(c) give the
+// acc[tn][tm][i] += sum_k X(m, k) W(n, k) over a (32 WT) x (32 WT) workgroup tile (WT = 2: 64 x 64,
+// WT = 4: 128 x 128 for large row counts). Wave quadrant: m = 16 WT * (wave >> 1) + 16 tm +
+// (lane & 15), n = 16 WT * (wave & 1) + 16 tn + 4 * (lane >> 4) + i; rowX(r) / rowW(c) give the
 // r-th X row / c-th W row of the tile.
-template <typename FX, typename FW>
-__device__ __forceinline__ void tile_mac_mfma(f32x4 (&acc)[2][2], FX rowX, FW rowW, int K, bf16 (*Xs)[MLD],
+// Workgroup barrier that orders LDS traffic only. __syncthreads() also drains every global load
+// in flight, which here are the next K step's prefetched segments: with it each K step would wait
+// out a full memory latency.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+}
+
+template <int WT, typename FX, typename FW>
+__device__ __forceinline__ void tile_mac_mfma(f32x4 (&acc)[WT][WT], FX rowX, FW rowW, int K, bf16 (*Xs)[MLD],
                                               bf16 (*Ws)[MLD]) {
+  constexpr int NS = WT / 2;                           // staged rows per thread and operand
   const int tid = threadIdx.x;
-  const int lr = tid >> 2, lk = (tid & 3) * 16;        // staging: row lr, k lk .. lk + 15
-  const RowRef rx = rowX(lr), rw = rowW(lr);
+  const int lr = tid >> 2, lk = (tid & 3) * 16;        // staging: rows lr + 64 j, k lk .. lk + 15
+  RowRef rx[NS], rw[NS];
+#pragma unroll
+  for (int j = 0; j < NS; ++j) {
+    rx[j] = rowX(lr + 64 * j);
+    rw[j] = rowW(lr + 64 * j);
+  }
   const int wave = tid >> 6, lane = tid & 63;
-  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32, r = lane & 15, g = lane >> 4;
-  bf16x8 x0 = load_row8(rx, lk, K), x1 = load_row8(rx, lk + 8, K);
-  bf16x8 w0 = load_row8(rw, lk, K), w1 = load_row8(rw, lk + 8, K);
+  const int wm = (wave >> 1) * 16 * WT, wn = (wave & 1) * 16 * WT, r = lane & 15, g = lane >> 4;
+  bf16x8 xv[NS][2], wv[NS][2];
+#pragma unroll
+  for (int j = 0; j < NS; ++j)
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      xv[j][e] = load_row8(rx[j], lk + 8 * e, K);
+      wv[j][e] = load_row8(rw[j], lk + 8 * e, K);
+    }
   for (int k0 = 0; k0 < K; k0 += MK) {
-    *reinterpret_cast<bf16x8*>(&Xs[lr][lk]) = x0;
-    *reinterpret_cast<bf16x8*>(&Xs[lr][lk + 8]) = x1;
-    *reinterpret_cast<bf16x8*>(&Ws[lr][lk]) = w0;
-    *reinterpret_cast<bf16x8*>(&Ws[lr][lk + 8]) = w1;
-    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NS; ++j)
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        *reinterpret_cast<bf16x8*>(&Xs[lr + 64 * j][lk + 8 * e]) = xv[j][e];
+        *reinterpret_cast<bf16x8*>(&Ws[lr + 64 * j][lk + 8 * e]) = wv[j][e];
+      }
+    lds_barrier();
     if (k0 + MK < K) {          // the next K step's segments travel while this one multiplies
-      x0 = load_row8(rx, k0 + MK + lk, K);
-      x1 = load_row8(rx, k0 + MK + lk + 8, K);
-      w0 = load_row8(rw, k0 + MK + lk, K);
-      w1 = load_row8(rw, k0 + MK + lk + 8, K);
+#pragma unroll
+      for (int j = 0; j < NS; ++j)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          xv[j][e] = load_row8(rx[j], k0 + MK + lk + 8 * e, K);
+          wv[j][e] = load_row8(rw[j], k0 + MK + lk + 8 * e, K);
+        }
     }
 #pragma unroll
     for (int ks = 0; ks < MK; ks += 32) {
-      bf16x8 xf[2], wf[2];
+      bf16x8 xf[WT], wf[WT];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
+      for (int t = 0; t < WT; ++t) {
         xf[t] = *reinterpret_cast<const bf16x8*>(&Xs[wm + 16 * t + r][ks + 8 * g]);
         wf[t] = *reinterpret_cast<const bf16x8*>(&Ws[wn + 16 * t + r][ks + 8 * g]);
       }
 #pragma unroll
-      for (int tn = 0; tn < 2; ++tn)
+      for (int tn = 0; tn < WT; ++tn)
 #pragma unroll
-        for (int tm = 0; tm < 2; ++tm) acc[tn][tm] = mfma16(wf[tn], xf[tm], acc[tn][tm]);
+        for (int tm = 0; tm < WT; ++tm) acc[tn][tm] = mfma16(wf[tn], xf[tm], acc[tn][tm]);
     }
-    __syncthreads();
+    lds_barrier();
   }
 }
 
-// f(m, n, value) over this lane's 16 results of the tile
-template <typename F>
-__device__ __forceinline__ void tile_each(const f32x4 (&acc)[2][2], F f) {
+// f(m, n, value) over this lane's results of the tile
+template <int WT, typename F>
+__device__ __forceinline__ void tile_each(const f32x4 (&acc)[WT][WT], F f) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+  const int wm = (wave >> 1) * 16 * WT, wn = (wave & 1) * 16 * WT;
 #pragma unroll
-  for (int tn = 0; tn < 2; ++tn)
+  for (int tn = 0; tn < WT; ++tn)
 #pragma unroll
-    for (int tm = 0; tm < 2; ++tm)
+    for (int tm = 0; tm < WT; ++tm)
 #pragma unroll
       for (int i = 0; i < 4; ++i) f(wm + 16 * tm + (lane & 15), wn + 16 * tn + 4 * (lane >> 4) + i, acc[tn][tm][i]);
 }
 
-#define BFLY_ZERO_ACC(a)                                   \
-  f32x4 a[2][2];                                           \
-  _Pragma("unroll") for (int _i = 0; _i < 2; ++_i)         \
-      _Pragma("unroll") for (int _j = 0; _j < 2; ++_j) a[_i][_j] = f32x4{0.f, 0.f, 0.f, 0.f}
+#define BFLY_ZERO_ACC(a)                                    \
+  f32x4 a[WT][WT];                                          \
+  _Pragma("unroll") for (int _i = 0; _i < WT; ++_i)         \
+      _Pragma("unroll") for (int _j = 0; _j < WT; ++_j) a[_i][_j] = f32x4{0.f, 0.f, 0.f, 0.f}
 
-template <typename TO>
+template <typename TO, int WT>
 __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(const bf16* __restrict__ x, long ldx,
                                                             const bf16* __restrict__ w, long ldw,
                                                             const bf16* __restrict__ bias, TO* __restrict__ out,
                                                             long ldo, int M, int N, int K, int act) {
-  __shared__ __attribute__((aligned(16))) bf16 Xs[TM][MLD], Ws[TN][MLD];
-  const int row0 = blockIdx.y * TM, col0 = blockIdx.x * TN;
+  constexpr int BT = 32 * WT;
+  __shared__ __attribute__((aligned(16))) bf16 Xs[BT][MLD], Ws[BT][MLD];
+  const int row0 = blockIdx.y * BT, col0 = blockIdx.x * BT;
   BFLY_ZERO_ACC(acc);
-  tile_mac_mfma(
+  tile_mac_mfma<WT>(
       acc, [&](int r) { return RowRef{row0 + r < M ? x + (long)(row0 + r) * ldx : nullptr, 1.f}; },
       [&](int c) { return RowRef{col0 + c < N ? w + (long)(col0 + c) * ldw : nullptr, 1.f}; }, K, Xs, Ws);
-  tile_each(acc, [&](int m, int n, float v) {
+  tile_each<WT>(acc, [&](int m, int n, float v) {
     const int r = row0 + m, c = col0 + n;
     if (r >= M || c >= N) return;
     if (bias) v += (float)bias[c];
@@ -379,6 +409,8 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(const bf16* __restri
   });
 }
 
+// `tiles` lists (expert, first row) of every (32 WT)-row tile of the grouped rows
+template <int WT>
 __global__ __launch_bounds__(256) void moe_glu_up_mfma_kernel(const bf16* __restrict__ x, long ldx,
                                                               const float* __restrict__ topk_w, int Kc,
                                                               const int* __restrict__ perm,
@@ -388,10 +420,11 @@ __global__ __launch_bounds__(256) void moe_glu_up_mfma_kernel(const bf16* __rest
                                                               const bf16* __restrict__ gu_w, float limit, float alpha,
                                                               bf16* __restrict__ hmid, int Hd, int F) {
   if ((int)blockIdx.y >= ntiles[0]) return;
-  __shared__ __attribute__((aligned(16))) bf16 Xs[TM][MLD], Ws[TN][MLD];
+  constexpr int BT = 32 * WT;
+  __shared__ __attribute__((aligned(16))) bf16 Xs[BT][MLD], Ws[BT][MLD];
   const int e = tiles[2 * blockIdx.y], r0 = tiles[2 * blockIdx.y + 1];
   const int rend = offsets_e[e + 1];
-  const int col0 = blockIdx.x * TN;
+  const int col0 = blockIdx.x * BT;
   const bf16* wg = gu_w + (long)e * 2 * F * Hd;
   const bf16* wu = wg + (long)F * Hd;
   // the expert's input row: the token row times its routing score, rounded to bf16
@@ -400,15 +433,17 @@ __global__ __launch_bounds__(256) void moe_glu_up_mfma_kernel(const bf16* __rest
     return p < 0 ? RowRef{nullptr, 1.f} : RowRef{x + (long)(p / Kc) * ldx, topk_w[p]};
   };
   BFLY_ZERO_ACC(g);
+  tile_mac_mfma<WT>(g, rowX, [&](int c) { return RowRef{col0 + c < F ? wg + (long)(col0 + c) * Hd : nullptr, 1.f}; },
+                    Hd, Xs, Ws);
   BFLY_ZERO_ACC(u);
-  tile_mac_mfma(g, rowX, [&](int c) { return RowRef{col0 + c < F ? wg + (long)(col0 + c) * Hd : nullptr, 1.f}; }, Hd, Xs, Ws);
-  tile_mac_mfma(u, rowX, [&](int c) { return RowRef{col0 + c < F ? wu + (long)(col0 + c) * Hd : nullptr, 1.f}; }, Hd, Xs, Ws);
+  tile_mac_mfma<WT>(u, rowX, [&](int c) { return RowRef{col0 + c < F ? wu + (long)(col0 + c) * Hd : nullptr, 1.f}; },
+                    Hd, Xs, Ws);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+  const int wm = (wave >> 1) * 16 * WT, wn = (wave & 1) * 16 * WT;
 #pragma unroll
-  for (int tn = 0; tn < 2; ++tn)
+  for (int tn = 0; tn < WT; ++tn)
 #pragma unroll
-    for (int tm = 0; tm < 2; ++tm)
+    for (int tm = 0; tm < WT; ++tm)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = r0 + wm + 16 * tm + (lane & 15), c = col0 + wn + 16 * tn + 4 * (lane >> 4) + i;
@@ -419,6 +454,7 @@ __global__ __launch_bounds__(256) void moe_glu_up_mfma_kernel(const bf16* __rest
       }
 }
 
+template <int WT>
 __global__ __launch_bounds__(256) void moe_down_mfma_kernel(const bf16* __restrict__ hmid, const int* __restrict__ perm,
                                                             const int* __restrict__ offsets_e,
                                                             const int* __restrict__ tiles,
@@ -426,16 +462,17 @@ __global__ __launch_bounds__(256) void moe_down_mfma_kernel(const bf16* __restri
                                                             const bf16* __restrict__ down_w, float* __restrict__ y,
                                                             int Hd, int F) {
   if ((int)blockIdx.y >= ntiles[0]) return;
-  __shared__ __attribute__((aligned(16))) bf16 Xs[TM][MLD], Ws[TN][MLD];
+  constexpr int BT = 32 * WT;
+  __shared__ __attribute__((aligned(16))) bf16 Xs[BT][MLD], Ws[BT][MLD];
   const int e = tiles[2 * blockIdx.y], r0 = tiles[2 * blockIdx.y + 1];
   const int rend = offsets_e[e + 1];
-  const int col0 = blockIdx.x * TN;
+  const int col0 = blockIdx.x * BT;
   const bf16* wd = down_w + (long)e * Hd * F;
   BFLY_ZERO_ACC(acc);
-  tile_mac_mfma(
+  tile_mac_mfma<WT>(
       acc, [&](int r) { return RowRef{r0 + r < rend ? hmid + (long)(r0 + r) * F : nullptr, 1.f}; },
       [&](int c) { return RowRef{col0 + c < Hd ? wd + (long)(col0 + c) * F : nullptr, 1.f}; }, F, Xs, Ws);
-  tile_each(acc, [&](int m, int n, float v) {
+  tile_each<WT>(acc, [&](int m, int n, float v) {
     const int r = r0 + m, c = col0 + n;
     if (r < rend && c < Hd) y[(long)perm[r] * Hd + c] = v;
   });
@@ -449,14 +486,24 @@ void launch_gemm_any(const void* x, long ldx, const void* w, long ldw, const voi
                      int M, int N, int K, int act, bool f32, bool out_f32, hipStream_t s) {
   if (M <= 0 || N <= 0) return;
   dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM);
+  if (!f32 && M >= 512 && N >= 128) {        // large row counts: the 128 x 128 workgroup tile
+    dim3 g2((N + 127) / 128, (M + 127) / 128);
+    if (out_f32)
+      gemm_any_mfma_kernel<float, 4><<<g2, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
+                                                        (float*)out, ldo, M, N, K, act);
+    else
+      gemm_any_mfma_kernel<bf16, 4><<<g2, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
+                                                       (bf16*)out, ldo, M, N, K, act);
+    return;
+  }
   if (f32)
     gemm_any_kernel<float, float><<<grid, 256, 0, s>>>((const float*)x, ldx, (const float*)w, ldw, (const float*)bias,
                                                        (float*)out, ldo, M, N, K, act);
   else if (out_f32)
-    gemm_any_mfma_kernel<float><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
+    gemm_any_mfma_kernel<float, 2><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
                                                      (float*)out, ldo, M, N, K, act);
   else
-    gemm_any_mfma_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
+    gemm_any_mfma_kernel<bf16, 2><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
                                                     (bf16*)out, ldo, M, N, K, act);
 }
 
@@ -474,30 +521,46 @@ void launch_moe_topk_scores(const float* logits, int top_k, int scoring, bool re
 
 int moe_sort_max_tiles(int TKp, int E) { return (TKp + 63) / 64 + E; }
 
-void launch_moe_sort(const int* ids, int TKp, int E, int* perm, int* offsets, int* tiles, int* ntiles, hipStream_t s) {
-  moe_sort_kernel<<<1, 1024, 0, s>>>(ids, TKp, E, perm, offsets, tiles, ntiles);
+// 128-row tiles when the experts average at least 256 grouped rows (bf16 only), else 64
+int moe_tile_rows(int TKp, int E, bool f32) { return (!f32 && TKp >= 256 * E) ? 128 : 64; }
+
+void launch_moe_sort(const int* ids, int TKp, int E, int* perm, int* offsets, int* tiles, int* ntiles, int tile_rows,
+                     hipStream_t s) {
+  moe_sort_kernel<<<1, 1024, 0, s>>>(ids, TKp, E, perm, offsets, tiles, ntiles, tile_rows);
 }
 
 void launch_moe_glu_up(const void* x, long ldx, const float* topk_w, int K, const int* perm, const int* offsets,
                        const int* tiles, const int* ntiles, int max_tiles, const void* gate_up_w, float limit,
-                       float alpha, void* hmid, int Hd, int F, bool f32, hipStream_t s) {
+                       float alpha, void* hmid, int Hd, int F, bool f32, int tile_rows, hipStream_t s) {
+  if (tile_rows == 128) {
+    dim3 g2((F + 127) / 128, max_tiles);
+    moe_glu_up_mfma_kernel<4><<<g2, 256, 0, s>>>((const bf16*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
+                                                 (const bf16*)gate_up_w, limit, alpha, (bf16*)hmid, Hd, F);
+    return;
+  }
   dim3 grid((F + TN - 1) / TN, max_tiles);
   if (f32)
     moe_glu_up_kernel<float><<<grid, 256, 0, s>>>((const float*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
                                                   (const float*)gate_up_w, limit, alpha, (float*)hmid, Hd, F);
   else
-    moe_glu_up_mfma_kernel<<<grid, 256, 0, s>>>((const bf16*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
+    moe_glu_up_mfma_kernel<2><<<grid, 256, 0, s>>>((const bf16*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
                                                 (const bf16*)gate_up_w, limit, alpha, (bf16*)hmid, Hd, F);
 }
 
 void launch_moe_down(const void* hmid, const int* perm, const int* offsets, const int* tiles, const int* ntiles,
-                     int max_tiles, const void* down_w, float* y, int Hd, int F, bool f32, hipStream_t s) {
+                     int max_tiles, const void* down_w, float* y, int Hd, int F, bool f32, int tile_rows, hipStream_t s) {
+  if (tile_rows == 128) {
+    dim3 g2((Hd + 127) / 128, max_tiles);
+    moe_down_mfma_kernel<4><<<g2, 256, 0, s>>>((const bf16*)hmid, perm, offsets, tiles, ntiles, (const bf16*)down_w, y,
+                                               Hd, F);
+    return;
+  }
   dim3 grid((Hd + TN - 1) / TN, max_tiles);
   if (f32)
     moe_down_kernel<float><<<grid, 256, 0, s>>>((const float*)hmid, perm, offsets, tiles, ntiles,
                                                 (const float*)down_w, y, Hd, F);
   else
-    moe_down_mfma_kernel<<<grid, 256, 0, s>>>((const bf16*)hmid, perm, offsets, tiles, ntiles, (const bf16*)down_w, y,
+    moe_down_mfma_kernel<2><<<grid, 256, 0, s>>>((const bf16*)hmid, perm, offsets, tiles, ntiles, (const bf16*)down_w, y,
                                               Hd, F);
 }
 

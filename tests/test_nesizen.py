@@ -74,7 +74,8 @@ def bf(t):
 # ---------------------------------------------------------------------------------------
 @pytest.mark.parametrize("M,N,K,bias,act", [(5, 7, 13, False, "none"), (70, 130, 50, True, "none"),
                                             (33, 64, 48, False, "relu2"), (1, 192, 256, True, "relu2"),
-                                            (130, 256, 128, False, "relu2")])
+                                            (130, 256, 128, False, "relu2"),
+                                            (600, 200, 130, True, "none"), (513, 129, 64, False, "relu2")])
 def test_linear_any_shape(target, M, N, K, bias, act):
     dev, dt = target
     g = torch.Generator().manual_seed(M * N + K)
@@ -266,11 +267,12 @@ def test_gla_output_norm_and_gate(target):
     assert (got.cpu().to(F64) - want).abs().max() < (1e-4 if dt == torch.float32 else 3e-2)
 
 
-@pytest.mark.parametrize("E,top,F,Hd", [(5, 2, 12, 40), (16, 1, 64, 64), (3, 3, 70, 24)])
-def test_sigmoid_router_and_glu_experts(target, E, top, F, Hd):
+@pytest.mark.parametrize("E,top,F,Hd,T", [(5, 2, 12, 40, 37), (16, 1, 64, 64, 37), (3, 3, 70, 24, 37),
+                                          (2, 2, 70, 136, 700)])      # the last: groups large enough for 128-row tiles
+def test_sigmoid_router_and_glu_experts(target, E, top, F, Hd, T):
     dev, dt = target
     g = torch.Generator().manual_seed(E * 10 + top)
-    T, limit = 37, 0.8
+    limit = 0.8
     x = bf(torch.randn(T, Hd, generator=g, dtype=F64))
     wr = bf(torch.randn(E, Hd, generator=g, dtype=F64) / math.sqrt(Hd) * 2)
     wg, wu = bf(torch.randn(E, F, Hd, generator=g, dtype=F64) / 3), bf(torch.randn(E, F, Hd, generator=g, dtype=F64) / 3)
