@@ -326,14 +326,14 @@ def cfg_c():
 
 def cfg_d():
     """Head sizes and widths that the MFMA kernels tile (bf16): attention 64 / 32 with a window of
-    40 and 6 kept tokens read again by a later layer with a longer window, GLA 64 / 64 and
-    32 / 128, two of eight experts."""
+    44 and 5 kept tokens, read again by a later layer with a longer window; GLA 64 / 64 and
+    32 / 128; two of eight experts; five streams."""
     return O.config([
-        O.gla_layer(2, 64, 64, 16.0, O.dense(256)),
-        O.attn_layer(4, 2, 64, 32, 32, 1e6, 0.125, 40, 6, O.moe(8, 2, 64, 1.0)),
+        O.gla_layer(2, 64, 64, 12.0, O.dense(256)),
+        O.attn_layer(4, 2, 64, 32, 32, 5e5, 0.11, 44, 5, O.moe(8, 2, 96, 1.5)),
         O.gla_layer(1, 32, 128, 4.0, None),
-        O.attn_layer(4, 2, 64, 32, 32, 1e6, 0.125, 70, 0, O.moe(8, 2, 64, 1.0), kv_from=1),
-    ], width=128, vocab=256, streams=3, eps=1e-6)
+        O.attn_layer(4, 2, 64, 32, 32, 5e5, 0.11, 70, 0, O.moe(8, 2, 96, 1.5), kv_from=1),
+    ], width=128, vocab=256, streams=5, eps=1e-5)
 
 
 _ORACLE = {}
