@@ -186,10 +186,14 @@ def layer_spec(index: int, L: dict) -> dict:
     sp = {"index": index, "type": t, "heads": int(m["heads"]), "dim": int(m["dim"]), "vdim": int(m["vdim"]),
           "kv_from": None, "kv_heads": 0}
     if t == "attention":
-        sp.update(kv_heads=int(m.get("kv_heads", m["heads"])), rot_dims=int(m["rot"]["dims"]),
-                  rot_base=float(m["rot"]["base"]), scale=float(m["scale"]), window=int(m["mask"]["size"]),
-                  keep_first=int(m["mask"].get("keep_first", 0)),
+        rot = m.get("rot") or {"dims": 0, "base": 10000.0}          # absent: no rotation
+        mask = m.get("mask") or {"size": 1 << 30}                    # absent: plain causal attention
+        sp.update(kv_heads=int(m.get("kv_heads", m["heads"])), rot_dims=int(rot["dims"]),
+                  rot_base=float(rot.get("base", 10000.0)), scale=float(m.get("scale", sp["dim"] ** -0.5)),
+                  window=int(mask["size"]), keep_first=int(mask.get("keep_first", 0)),
                   kv_from=None if m.get("kv_from") is None else int(m["kv_from"]))
+        if sp["window"] < 1 or sp["keep_first"] < 0:
+            raise ValueError(f"layer {index}: window must be >= 1 and keep_first >= 0")
         if sp["heads"] % sp["kv_heads"] or sp["rot_dims"] % 2 or sp["rot_dims"] > sp["dim"]:
             raise ValueError(f"layer {index}: bad attention sizes")
     elif t == "gla":
