@@ -370,6 +370,75 @@ __device__ __forceinline__ void tile_mac_mfma(f32x4 (&acc)[WT][WT], FX rowX, FW 
   }
 }
 
+// tile_mac_mfma for two weight panels that share the X tile (an expert's gate and up rows): one K
+// loop, X staged once, both panels' segments in flight together.
+template <int WT, typename FX, typename FW, typename FV>
+__device__ __forceinline__ void tile_mac_mfma2(f32x4 (&acc)[WT][WT], f32x4 (&acc2)[WT][WT], FX rowX, FW rowW, FV rowV,
+                                               int K, bf16 (*Xs)[MLD], bf16 (*Ws)[MLD], bf16 (*Vs)[MLD]) {
+  constexpr int NS = WT / 2;
+  const int tid = threadIdx.x;
+  const int lr = tid >> 2, lk = (tid & 3) * 16;
+  RowRef rx[NS], rw[NS], rv[NS];
+#pragma unroll
+  for (int j = 0; j < NS; ++j) {
+    rx[j] = rowX(lr + 64 * j);
+    rw[j] = rowW(lr + 64 * j);
+    rv[j] = rowV(lr + 64 * j);
+  }
+  const int wave = tid >> 6, lane = tid & 63;
+  const int wm = (wave >> 1) * 16 * WT, wn = (wave & 1) * 16 * WT, r = lane & 15, g = lane >> 4;
+  bf16x8 xv[NS][2], wv[NS][2], vv[NS][2];
+#pragma unroll
+  for (int j = 0; j < NS; ++j)
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      xv[j][e] = load_row8(rx[j], lk + 8 * e, K);
+      wv[j][e] = load_row8(rw[j], lk + 8 * e, K);
+      vv[j][e] = load_row8(rv[j], lk + 8 * e, K);
+    }
+  for (int k0 = 0; k0 < K; k0 += MK) {
+#pragma unroll
+    for (int j = 0; j < NS; ++j)
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        *reinterpret_cast<bf16x8*>(&Xs[lr + 64 * j][lk + 8 * e]) = xv[j][e];
+        *reinterpret_cast<bf16x8*>(&Ws[lr + 64 * j][lk + 8 * e]) = wv[j][e];
+        *reinterpret_cast<bf16x8*>(&Vs[lr + 64 * j][lk + 8 * e]) = vv[j][e];
+      }
+    lds_barrier();
+    if (k0 + MK < K) {
+#pragma unroll
+      for (int j = 0; j < NS; ++j)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          xv[j][e] = load_row8(rx[j], k0 + MK + lk + 8 * e, K);
+          wv[j][e] = load_row8(rw[j], k0 + MK + lk + 8 * e, K);
+          vv[j][e] = load_row8(rv[j], k0 + MK + lk + 8 * e, K);
+        }
+    }
+#pragma unroll
+    for (int ks = 0; ks < MK; ks += 32) {
+      bf16x8 xf[WT], wf[WT];
+#pragma unroll
+      for (int t = 0; t < WT; ++t) {
+        xf[t] = *reinterpret_cast<const bf16x8*>(&Xs[wm + 16 * t + r][ks + 8 * g]);
+        wf[t] = *reinterpret_cast<const bf16x8*>(&Ws[wn + 16 * t + r][ks + 8 * g]);
+      }
+#pragma unroll
+      for (int tn = 0; tn < WT; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < WT; ++tm) acc[tn][tm] = mfma16(wf[tn], xf[tm], acc[tn][tm]);
+#pragma unroll
+      for (int t = 0; t < WT; ++t) wf[t] = *reinterpret_cast<const bf16x8*>(&Vs[wn + 16 * t + r][ks + 8 * g]);
+#pragma unroll
+      for (int tn = 0; tn < WT; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < WT; ++tm) acc2[tn][tm] = mfma16(wf[tn], xf[tm], acc2[tn][tm]);
+    }
+    lds_barrier();
+  }
+}
+
 // f(m, n, value) over this lane's results of the tile
 template <int WT, typename F>
 __device__ __forceinline__ void tile_each(const f32x4 (&acc)[WT][WT], F f) {
@@ -421,7 +490,10 @@ __global__ __launch_bounds__(256) void moe_glu_up_mfma_kernel(const bf16* __rest
                                                               bf16* __restrict__ hmid, int Hd, int F) {
   if ((int)blockIdx.y >= ntiles[0]) return;
   constexpr int BT = 32 * WT;
-  __shared__ __attribute__((aligned(16))) bf16 Xs[BT][MLD], Ws[BT][MLD];
+  // small groups (decode): gate and up share one K loop, so both panels' weight segments are in
+  // flight together; large groups (128-row tiles): two passes, which keep registers and LDS for
+  // a second resident workgroup
+  __shared__ __attribute__((aligned(16))) bf16 Xs[BT][MLD], Ws[BT][MLD], Vs[WT == 2 ? BT : 1][MLD];
   const int e = tiles[2 * blockIdx.y], r0 = tiles[2 * blockIdx.y + 1];
   const int rend = offsets_e[e + 1];
   const int col0 = blockIdx.x * BT;
@@ -433,11 +505,15 @@ __global__ __launch_bounds__(256) void moe_glu_up_mfma_kernel(const bf16* __rest
     return p < 0 ? RowRef{nullptr, 1.f} : RowRef{x + (long)(p / Kc) * ldx, topk_w[p]};
   };
   BFLY_ZERO_ACC(g);
-  tile_mac_mfma<WT>(g, rowX, [&](int c) { return RowRef{col0 + c < F ? wg + (long)(col0 + c) * Hd : nullptr, 1.f}; },
-                    Hd, Xs, Ws);
   BFLY_ZERO_ACC(u);
-  tile_mac_mfma<WT>(u, rowX, [&](int c) { return RowRef{col0 + c < F ? wu + (long)(col0 + c) * Hd : nullptr, 1.f}; },
-                    Hd, Xs, Ws);
+  auto rowG = [&](int c) { return RowRef{col0 + c < F ? wg + (long)(col0 + c) * Hd : nullptr, 1.f}; };
+  auto rowU = [&](int c) { return RowRef{col0 + c < F ? wu + (long)(col0 + c) * Hd : nullptr, 1.f}; };
+  if constexpr (WT == 2) {
+    tile_mac_mfma2<WT>(g, u, rowX, rowG, rowU, Hd, Xs, Ws, Vs);
+  } else {
+    tile_mac_mfma<WT>(g, rowX, rowG, Hd, Xs, Ws);
+    tile_mac_mfma<WT>(u, rowX, rowU, Hd, Xs, Ws);
+  }
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = (wave >> 1) * 16 * WT, wn = (wave & 1) * 16 * WT;
 #pragma unroll
