@@ -860,8 +860,13 @@ def moe_route_scores(x, wr, top_k: int, scoring: str = "softmax", renorm: bool =
     if not _gpu(x):
         return ref.moe_route_scores(x, wr, top_k, scoring, renorm)
     T = x.shape[0]
-    # logits: a GEMM with f32 accumulation and f32 output, then one wave per token picks
-    logits = linear_act(x, wr, out_dtype=torch.float32)
+    # logits: a GEMM with f32 accumulation and f32 output (steps of a few rows: one wave per
+    # (token, expert) instead of a one-workgroup GEMM), then one wave per token picks
+    if T * wr.shape[0] <= 4096:
+        logits = _empty(T, wr.shape[0], dtype=torch.float32, device=x.device)
+        torch.ops.bfly.router_logits(x, wr, logits)
+    else:
+        logits = linear_act(x, wr, out_dtype=torch.float32)
     ids = _empty(T, top_k, dtype=torch.int32, device=x.device)
     w = _empty(T, top_k, dtype=torch.float32, device=x.device)
     torch.ops.bfly.moe_topk_scores(logits, top_k, {"softmax": 0, "sigmoid": 1}[scoring], bool(renorm), ids, w)

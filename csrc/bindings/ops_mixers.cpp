@@ -217,6 +217,15 @@ void gla_out(const Tensor& o, const Tensor& g, const Tensor& norm_w, double eps,
                        out.data_ptr(), (int)T, (int)H, (int)Dv, is_f32(out), cur_stream());
 }
 
+void router_logits(const Tensor& x, const Tensor& wr, Tensor& logits) {
+  CHK_GPU(x); CHK_SAME(x, wr); CHK_F32(logits);
+  TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1 && wr.dim() == 2 && wr.is_contiguous(), "router_logits: layouts");
+  const int64_t T = x.size(0), Hd = x.size(1), E = wr.size(0);
+  TORCH_CHECK(wr.size(1) == Hd && logits.dim() == 2 && logits.size(0) == T && logits.size(1) == E, "router_logits: shapes");
+  bfly::launch_router_logits(x.data_ptr(), x.stride(0), wr.data_ptr(), logits.data_ptr<float>(), (int)T, (int)E, (int)Hd,
+                             is_f32(x), cur_stream());
+}
+
 void moe_topk_scores(const Tensor& logits, int64_t top_k, int64_t scoring, bool renorm, Tensor& ids, Tensor& w) {
   CHK_GPU(logits); CHK_F32(logits); CHK_I32(ids); CHK_F32(w);
   TORCH_CHECK(logits.dim() == 2, "moe_topk_scores: logits [T, E]");
@@ -292,6 +301,7 @@ TORCH_LIBRARY_FRAGMENT(bfly, m) {
   m.def("gla_scan(Tensor q, Tensor k, Tensor v, Tensor z, Tensor(a!) state, Tensor state_slots, Tensor row_cu, "
         "Tensor positions, float tau, float q_scale, Tensor(b!) o) -> ()");
   m.def("gla_out(Tensor o, Tensor g, Tensor norm_w, float eps, Tensor(a!) out) -> ()");
+  m.def("router_logits(Tensor x, Tensor wr, Tensor(a!) logits) -> ()");
   m.def("moe_topk_scores(Tensor logits, int top_k, int scoring, bool renorm, Tensor(a!) ids, Tensor(b!) w) -> ()");
   m.def("moe_sort_max_tiles(int tk, int experts) -> int", &moe_sort_max_tiles);
   m.def("moe_glu_ffn(Tensor x, Tensor topk_ids, Tensor topk_w, Tensor gate_up_w, Tensor down_w, float limit, "
@@ -312,6 +322,7 @@ TORCH_LIBRARY_IMPL(bfly, CUDA, m) {
   m.impl("attn_window_paged", &attn_window_paged);
   m.impl("gla_scan", &gla_scan);
   m.impl("gla_out", &gla_out);
+  m.impl("router_logits", &router_logits);
   m.impl("moe_topk_scores", &moe_topk_scores);
   m.impl("moe_glu_ffn", &moe_glu_ffn);
 }

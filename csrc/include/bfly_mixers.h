@@ -67,6 +67,9 @@ int launch_gla_scan(const void* q, long q_ld, const void* k, long k_ld, const vo
 void launch_gla_out(const float* o, const void* g, long g_ld, const float* norm_w, float eps, void* out, int T, int H,
                     int Dv, bool f32, hipStream_t s);
 
+// logits[t, e] = x[t] . wr[e] in f32, one wave per pair (for steps of a few rows)
+void launch_router_logits(const void* x, long ldx, const void* wr, float* logits, int T, int E, int Hd, bool f32,
+                          hipStream_t s);
 // Router choice from f32 logits [T, E]: scoring 0 softmax / 1 sigmoid, top-k (ties: lowest id),
 // optional renorm. E <= 1024.
 void launch_moe_topk_scores(const float* logits, int top_k, int scoring, bool renorm, int* ids, float* w, int T, int E,

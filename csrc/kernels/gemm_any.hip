@@ -219,6 +219,22 @@ __global__ void moe_sum_kernel(const float* __restrict__ y, int Kc, T* __restric
   }
 }
 
+// Router logits of a small step (a few rows): one wave per (token, expert), lanes split the
+// hidden dim, f32 accumulation. Large steps use the f32-output GEMM instead.
+template <typename T>
+__global__ __launch_bounds__(256) void router_logits_kernel(const T* __restrict__ x, long ldx,
+                                                            const T* __restrict__ wr, float* __restrict__ logits,
+                                                            int E, int Hd) {
+  const int t = blockIdx.x, e = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (e >= E) return;
+  const T* xr = x + (long)t * ldx;
+  const T* w = wr + (long)e * Hd;
+  float a = 0.f;
+  for (int k = lane; k < Hd; k += 64) a = fmaf(ldf(xr + k), ldf(w + k), a);
+  a = wave_sum(a);
+  if (lane == 0) logits[(long)t * E + e] = a;
+}
+
 // Router choice of one token per wave from its f32 logits [E]: softmax or sigmoid scores, K rounds
 // of arg-max over the experts (ties to the lowest id).
 __global__ __launch_bounds__(64) void moe_topk_scores_kernel(const float* __restrict__ logits, int top_k, int scoring,
@@ -587,6 +603,14 @@ void launch_relu2(void* x, long n, bool f32, hipStream_t s) {
   if (n <= 0) return;
   if (f32) relu2_kernel<float><<<ew_blocks(n), 256, 0, s>>>((float*)x, n);
   else relu2_kernel<bf16><<<ew_blocks(n), 256, 0, s>>>((bf16*)x, n);
+}
+
+void launch_router_logits(const void* x, long ldx, const void* wr, float* logits, int T, int E, int Hd, bool f32,
+                          hipStream_t s) {
+  if (T <= 0) return;
+  dim3 grid(T, (E + 3) / 4);
+  if (f32) router_logits_kernel<float><<<grid, 256, 0, s>>>((const float*)x, ldx, (const float*)wr, logits, E, Hd);
+  else router_logits_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)wr, logits, E, Hd);
 }
 
 void launch_moe_topk_scores(const float* logits, int top_k, int scoring, bool renorm, int* ids, float* w, int T, int E,
