@@ -16,7 +16,7 @@ from typing import Any, Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str                       # "llama" | "gpt2" | "mixtral" | "nesizen"
+    arch: str                       # "llama" | "gpt2" | "mixtral" | "nesizen" | "zinesun"
     vocab_size: int
     hidden_size: int
     intermediate_size: int
@@ -40,6 +40,8 @@ class ModelConfig:
     # the flat fields above then hold the largest value over the layers (workspace sizing)
     layer_specs: Optional[list] = None
     residual_streams: int = 1       # > 1: hyper-connections (parallel residual streams)
+    embed_scale: float = 1.0        # the embedding rows are multiplied by this
+    conv_taps: int = 0              # > 1: causal per-channel convolution over time on a mixer's input
 
     # ---- derived quantities ------------------------------------------------------------
     @property
@@ -88,8 +90,12 @@ class ModelConfig:
 
     def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
         if self.layer_specs:
+            # a latent-attention layer caches its latent twice (key rows and transposed value
+            # rows) and the shared rotated key part once
             return sum(sp["kv_heads"] * (sp["dim"] + sp["vdim"]) * dtype_bytes for sp in self.layer_specs
-                       if sp["type"] == "attention" and sp["kv_from"] is None)
+                       if sp["type"] == "attention" and sp["kv_from"] is None) + \
+                sum((2 * sp["kv_rank"] + sp["rot_dim"]) * dtype_bytes for sp in self.layer_specs
+                    if sp["type"] == "latent_attention")
         return 2 * self.num_layers * self.kv_size * dtype_bytes
 
     # ---- (de)serialisation -------------------------------------------------------------
@@ -134,13 +140,39 @@ class ModelConfig:
                    layer_specs=specs, residual_streams=int(js.get("streams", 1)))
 
     @classmethod
+    def from_zinesun(cls, js: dict, name: str = "zinesun") -> "ModelConfig":
+        """Map a Zinesun config.json ("architecture": "Zinesun") to ModelConfig: latent-attention
+        layers with dense or routed feed-forwards, post-sublayer layer norms, a causal convolution
+        on every mixer's input and a learned average over the outputs of all earlier layers. Every
+        size and per-layer constant is taken from the file."""
+        specs = [layer_spec(i, L) for i, L in enumerate(js["layers"])]
+        mx = lambda key: max([sp.get(key) or 0 for sp in specs] + [0])  # noqa: E731
+        moe = [sp["ffn"] for sp in specs if sp["ffn"] and sp["ffn"]["kind"] == "moe"]
+        taps = int((js.get("canon") or {}).get("taps", 0))
+        if taps < 0:
+            raise ValueError("canon.taps must be >= 0")
+        return cls(name=name, arch="zinesun", vocab_size=int(js["vocab"]), hidden_size=int(js["width"]),
+                   intermediate_size=max([sp["ffn"]["ff"] for sp in specs if sp["ffn"]] + [0]),
+                   num_layers=len(specs), num_heads=mx("heads"), num_kv_heads=1,
+                   head_dim=max(mx("kv_rank") + mx("rot_dim"), mx("dim") + mx("rot_dim"), mx("vdim")),
+                   max_position=1 << 30, norm_eps=float(js["norm"]["eps"]),
+                   norm="layer", act="xielu", pos_emb="rope", tie_embeddings=True,
+                   num_experts=max([m["experts"] for m in moe] + [0]),
+                   experts_per_token=max([m["top"] for m in moe] + [0]),
+                   layer_specs=specs, embed_scale=float((js.get("embedding") or {}).get("scale", 1.0)),
+                   conv_taps=taps)
+
+    @classmethod
     def from_model_dir(cls, path, name: Optional[str] = None) -> "ModelConfig":
         """config.json of a model folder -> ModelConfig; the "architecture" / "model_type" key
         chooses the family."""
         js = json.loads((Path(path) / "config.json").read_text())
         name = name or Path(path).name
-        if str(js.get("architecture", "")).lower() == "nesizen":
+        family = str(js.get("architecture", "")).lower()
+        if family == "nesizen":
             return cls.from_nesizen(js, name=name)
+        if family == "zinesun":
+            return cls.from_zinesun(js, name=name)
         return cls.from_hf(js, name=name)
 
     @classmethod
@@ -180,8 +212,11 @@ class ModelConfig:
 def layer_spec(index: int, L: dict) -> dict:
     """One layer of a heterogeneous stack, normalised to flat keys. `type` "attention": windowed
     softmax attention (heads, kv_heads, dim, vdim, rot_dims, rot_base, scale, window, keep_first,
-    kv_from); "gla": gated linear attention (heads, dim, vdim, tau). `ffn`: None, or kind
-    "dense" (ff) / "moe" (ff, limit, experts, top)."""
+    kv_from); "latent_attention": windowed softmax attention whose queries, keys and values are
+    expanded from low-rank latents, with one rotated key part shared by the heads (heads, dim,
+    rot_dim, vdim, kv_rank, q_rank, rot_base, scale, window); "gla": gated linear attention
+    (heads, dim, vdim, tau). `ffn`: None, or kind "dense" (ff) / "moe" (ff, limit or None for
+    unclamped experts, experts, top)."""
     m, t = L["mixer"], L["type"]
     sp = {"index": index, "type": t, "heads": int(m["heads"]), "dim": int(m["dim"]), "vdim": int(m["vdim"]),
           "kv_from": None, "kv_heads": 0}
@@ -196,6 +231,17 @@ def layer_spec(index: int, L: dict) -> dict:
             raise ValueError(f"layer {index}: window must be >= 1 and keep_first >= 0")
         if sp["heads"] % sp["kv_heads"] or sp["rot_dims"] % 2 or sp["rot_dims"] > sp["dim"]:
             raise ValueError(f"layer {index}: bad attention sizes")
+    elif t == "latent_attention":
+        rot = m.get("rot") or {}
+        mask = m.get("mask") or {"size": 1 << 30}
+        sp.update(rot_dim=int(m.get("rot_dim", 0)), kv_rank=int(m["kv_rank"]), q_rank=int(m["q_rank"]),
+                  rot_base=float(rot.get("base", 10000.0)),
+                  scale=float(m.get("scale", (sp["dim"] + int(m.get("rot_dim", 0))) ** -0.5)),
+                  window=int(mask["size"]))
+        if int(rot.get("dims", sp["rot_dim"])) != sp["rot_dim"]:
+            raise ValueError(f"layer {index}: the rotated part is rot_dim wide (rot.dims must equal it)")
+        if sp["window"] < 1 or sp["rot_dim"] % 2 or min(sp["kv_rank"], sp["q_rank"], sp["dim"] + sp["rot_dim"]) < 1:
+            raise ValueError(f"layer {index}: bad latent-attention sizes")
     elif t == "gla":
         sp.update(tau=float(m["tau"]))
     else:
@@ -206,7 +252,8 @@ def layer_spec(index: int, L: dict) -> dict:
     elif f["kind"] == "dense":
         sp["ffn"] = {"kind": "dense", "ff": int(f["ff"])}
     elif f["kind"] == "moe":
-        sp["ffn"] = {"kind": "moe", "ff": int(f["expert"]["ff"]), "limit": float(f["expert"]["limit"]),
+        lim = f["expert"].get("limit")
+        sp["ffn"] = {"kind": "moe", "ff": int(f["expert"]["ff"]), "limit": None if lim is None else float(lim),
                      "experts": int(f["router"]["experts"]), "top": int(f["router"]["top"])}
         if not 1 <= sp["ffn"]["top"] <= sp["ffn"]["experts"]:
             raise ValueError(f"layer {index}: top must be in 1..experts")
@@ -221,6 +268,9 @@ def layer_spec_params(h: int, sp: dict) -> int:
         n = h * H * D + H * Dv * h + H
         if sp["kv_from"] is None:
             n += h * sp["kv_heads"] * (D + Dv)
+    elif sp["type"] == "latent_attention":
+        R, Q, rd = sp["kv_rank"], sp["q_rank"], sp["rot_dim"]
+        n = h * (Q + R + rd + H) + Q + R + Q * H * (D + rd) + R * H * (D + Dv) + H * Dv * h
     else:
         n = h * H * (2 * D + 2 * Dv) + H * Dv * h + Dv
     f = sp["ffn"]

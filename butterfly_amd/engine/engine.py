@@ -34,7 +34,7 @@ import torch
 
 from .. import ops
 from ..config import EngineConfig, ModelConfig
-from ..models import Shard, build_model
+from ..models import Shard, build_model, supports_f32
 from ..parallel.comm import Communicator, NativeWork
 from ..parallel.mesh import Mesh
 from ..partition.plan import PartitionPlan
@@ -123,7 +123,7 @@ class LLMEngine:
         # kernels have an f32 form; the bf16-only families refuse it on the GPU)
         want32 = str(engine_cfg.dtype).lower() in ("fp32", "float32", "f32")
         dtype = torch.float32 if (self.device.type != "cuda" or want32) else torch.bfloat16
-        if want32 and self.device.type == "cuda" and model is None and cfg.arch != "nesizen":
+        if want32 and self.device.type == "cuda" and model is None and not supports_f32(cfg.arch):
             raise NotImplementedError(f"{cfg.arch} GPU kernels are bf16 only (EngineConfig.dtype = 'bf16')")
         self.model = model or build_model(cfg, shard, device=self.device, dtype=dtype, comm=self.comm)
         if model is None:

@@ -1,8 +1,10 @@
 """Model families: Llama-3 (8B/70B), Mixtral 8x7B (MoE), GPT-2 — one shard-aware decoder — and
-Nesizen, a heterogeneous stack of attention / gated-linear-attention layers (models/nesizen.py)."""
+Nesizen, a heterogeneous stack of attention / gated-linear-attention layers (models/nesizen.py),
+and Zinesun, latent-attention layers on a post-norm residual (models/zinesun.py)."""
 from .shard import LocalDims, Shard, local_dims  # noqa: F401
 from .transformer import LogicalParam, TransformerLM  # noqa: F401
 from .nesizen import NesizenLM  # noqa: F401
+from .zinesun import ZinesunLM  # noqa: F401
 
 
 class LlamaForCausalLM(TransformerLM):
@@ -18,7 +20,12 @@ class GPT2LMHeadModel(TransformerLM):
 
 
 _ARCH = {"llama": LlamaForCausalLM, "mixtral": MixtralForCausalLM, "gpt2": GPT2LMHeadModel,
-         "nesizen": NesizenLM}
+         "nesizen": NesizenLM, "zinesun": ZinesunLM}
+
+
+def supports_f32(arch: str) -> bool:
+    """Whether the family's GPU kernels have a true 32-bit form (EngineConfig.dtype = "fp32")."""
+    return bool(getattr(_ARCH[arch], "supports_f32", False))
 
 
 def build_model(cfg, shard=None, device="cpu", dtype=None, comm=None):

@@ -37,20 +37,15 @@ from ..config import ModelConfig
 from ..engine.batch import ForwardBatch
 from ..parallel.comm import Communicator
 from .shard import LocalDims, Shard
+from .stack import PackedStack, pad128 as _pad128
 from .transformer import LogicalParam, _name_seed
-
-def _pad128(n: int) -> int:
-    """Fused projections carry zero rows up to a multiple of 128 (the MFMA GEMMs' N tiling)."""
-    return (n + 127) // 128 * 128
 
 
 NORM_OFFSET = 1.0       # norm weights are stored around zero
 GLU_ALPHA = 1.702       # expert activation g * sigmoid(alpha g)
 
 
-class NesizenLM:
-    paged_prefill_only = True     # the runner builds block tables for every prompt chunk
-
+class NesizenLM(PackedStack):
     def __init__(self, cfg: ModelConfig, shard: Shard = Shard(), device="cpu",
                  dtype: torch.dtype = torch.bfloat16, comm: Optional[Communicator] = None):
         if not cfg.layer_specs:
@@ -155,15 +150,6 @@ class NesizenLM:
     def head_weight(self) -> torch.Tensor:
         return self.p["head"]
 
-    def local_bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in self.p.values() if t is not None)
-
-    def packed_decode_bytes(self, kinds=None) -> int:
-        return 0
-
-    def pack_decode_weights(self, budget_bytes=None, kinds=None) -> int:
-        return 0
-
     def logical_params(self) -> list[LogicalParam]:
         """Checkpoint tensors by their file names ('l<i>.mix.q', 'l<i>.mlp.e<j>.gate', ...), each
         a view into the fused local tensors."""
@@ -255,10 +241,6 @@ class NesizenLM:
     # ------------------------------------------------------------------------------------
     # caches
     # ------------------------------------------------------------------------------------
-    def kv_bytes_per_token(self, dtype: Optional[torch.dtype] = None) -> int:
-        es = torch.empty((), dtype=dtype or self.dtype).element_size()
-        return max(1, self.cfg.kv_bytes_per_token(es))
-
     def state_bytes_per_slot(self) -> int:
         return sum(4 * sp["heads"] * sp["dim"] * sp["vdim"] for sp in self.specs if sp["type"] == "gla")
 
@@ -282,42 +264,9 @@ class NesizenLM:
                       for sp in self.specs if sp["type"] == "gla"]
         return self.state
 
-    def gemm_shapes(self) -> list:
-        return sorted({tuple(w.shape) for k, w in self.p.items()
-                       if w is not None and w.dim() == 2 and w.dtype == torch.bfloat16 and k != "embed"
-                       and w.shape[0] % 128 == 0 and w.shape[1] % 64 == 0})
-
     # ------------------------------------------------------------------------------------
     # forward
     # ------------------------------------------------------------------------------------
-    def _iota(self, n: int) -> torch.Tensor:
-        t = self._arange.get(n)
-        if t is None:
-            t = self._arange[n] = torch.arange(n, dtype=torch.int32, device=self.device)
-        return t
-
-    def _step_meta(self, fb: ForwardBatch) -> dict:
-        """Packed-row description shared by the mixers: row_cu [nseq + 1] (decode rows are
-        one-row sequences, then the prompt chunks), one block table per sequence, state slots."""
-        T = fb.num_tokens
-        if not fb.is_prefill:
-            row_cu, tables = self._iota(T + 1), fb.block_tables
-        else:
-            nd = fb.num_decode
-            if fb.cu_seqlens.numel() > 1 and fb.prefix_tables is None:
-                raise RuntimeError("Nesizen prompt chunks need their block tables (mixed scheduling)")
-            if nd:
-                row_cu = torch.cat([self._iota(nd), fb.cu_seqlens + nd])
-                tables = fb.block_tables[:nd] if fb.prefix_tables is None else torch.cat([fb.block_tables[:nd], fb.prefix_tables])
-            else:
-                row_cu, tables = fb.cu_seqlens, fb.prefix_tables
-        m = {"row_cu": row_cu, "tables": tables, "state_slots": fb.state_slots, "row_map": None}
-        if self.has_state and fb.state_slots is None and T:
-            raise RuntimeError("Nesizen needs the batch's recurrent-state slots")
-        if self.device.type == "cuda" and T and any(sp["type"] == "attention" for sp in self.specs):
-            m["row_map"] = ops.row_seq(row_cu, T)
-        return m
-
     def forward(self, fb: ForwardBatch, kv_caches: Optional[list] = None,
                 hidden_in: Optional[torch.Tensor] = None) -> torch.Tensor:
         """One step over the packed rows of `fb`; returns logits [R, padded vocab] for the rows
@@ -385,4 +334,5 @@ class NesizenLM:
         if fs["kind"] == "dense":
             return ops.linear_act(ops.linear_act(h, self.p[pre + "up"], act="relu2"), self.p[pre + "down"])
         ids, w = ops.moe_route_scores(h, self.p[pre + "router"], fs["top"], scoring="sigmoid", renorm=False)
-        return ops.moe_glu_ffn(h, ids, w, self.p[pre + "gate_up"], self.p[pre + "edown"], fs["limit"], GLU_ALPHA)
+        return ops.moe_glu_ffn(h, ids, w, self.p[pre + "gate_up"], self.p[pre + "edown"],
+                               float("inf") if fs["limit"] is None else fs["limit"], GLU_ALPHA)

@@ -729,7 +729,7 @@ def moe_gate_scale_(h, gates, e0: int, num_local: int):
 # ---------------------------------------------------------------------------------------
 # Shape-generic ops (csrc/kernels/gemm_any.hip, hyper.hip, mixers.hip): bf16 or f32 tensors
 # ---------------------------------------------------------------------------------------
-ACTS = {"none": 0, "relu2": 1}
+ACTS = {"none": 0, "relu2": 1, "xielu": 2}
 
 
 def _mfma_gemm_ok(x, w, out_dtype) -> bool:
@@ -738,19 +738,22 @@ def _mfma_gemm_ok(x, w, out_dtype) -> bool:
             and w.shape[0] % 128 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and x.shape[0] > 0)
 
 
-def linear_act(x, w, bias=None, act: str = "none", out_dtype=None):
+def linear_act(x, w, bias=None, act: str = "none", out_dtype=None, act_params=None):
     """y = act(x w^T + bias) for any shape, bf16 or f32 (`out_dtype` f32: keep the f32
-    accumulator). bf16 shapes the MFMA GEMMs tile go to them (the activation as a pass over the
-    result); every other shape, and f32, runs the generic tile kernel."""
+    accumulator). act: "none" | "relu2" | "xielu" (act_params = its two coefficients (a_pos,
+    a_neg): z > 0: a_pos z^2 + z / 2, else a_neg (exp(z) - 1 - z) + z / 2). bf16 shapes the MFMA
+    GEMMs tile go to them (the activation as a pass over the result); every other shape, and f32,
+    runs the generic tile kernel."""
     if not _gpu(x):
-        return ref.linear_act(x, w, bias, act, out_dtype)
+        return ref.linear_act(x, w, bias, act, out_dtype, act_params)
+    a0, a1 = (float(act_params[0]), float(act_params[1])) if act == "xielu" else (0.0, 0.0)
     if _mfma_gemm_ok(x, w, out_dtype):
         y = linear(x, w, bias=bias)
-        if act == "relu2":
-            torch.ops.bfly.relu2_(y)
+        if act != "none":
+            torch.ops.bfly.act_(y, ACTS[act], a0, a1)
         return y
     out = _empty(x.shape[0], w.shape[0], dtype=out_dtype or x.dtype, device=x.device)
-    torch.ops.bfly.gemm_any(x, w, bias, ACTS[act], out)
+    torch.ops.bfly.gemm_any(x, w, bias, ACTS[act], a0, a1, out)
     return out
 
 
@@ -821,18 +824,22 @@ def row_seq(row_cu, T: int):
 
 
 def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale: float, window: int, keep_first: int,
-                      sink, row_map=None, out=None):
+                      sink, row_map=None, out=None, fold_heads: bool = False, out_scale=None):
     """Windowed attention of packed rows over the paged cache with kept first positions and a
-    sink logit (mixers.hip attn_window_paged_kernel). `row_map`: ops.row_seq(row_cu, T), when the
-    caller already has it."""
+    sink logit (mixers.hip attn_window_paged_kernel; sink None: an ordinary softmax). `row_map`:
+    ops.row_seq(row_cu, T), when the caller already has it. `out_scale` [T, H] f32 multiplies
+    every head's output (an output gate). `fold_heads` (one shared key / value head only): the
+    heads of a token become rows of the attention tiles, so a token's heads read each cached
+    page once instead of once per head."""
     if not _gpu(q):
-        return ref.attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, window, keep_first, sink, out)
+        return ref.attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, window, keep_first, sink, out,
+                                     out_scale)
     if out is None:
         out = _empty(q.shape[0], q.shape[1], v_cache.shape[2], dtype=q.dtype, device=q.device)
     if row_map is None:
         row_map = row_seq(row_cu, q.shape[0])
     torch.ops.bfly.attn_window_paged(q, k_cache, v_cache, tables, row_map, row_cu, positions, float(scale), int(window),
-                                     int(keep_first), sink, out)
+                                     int(keep_first), sink, out_scale, bool(fold_heads), out)
     return out
 
 
@@ -854,11 +861,12 @@ def gla_out(o, g, norm_w, eps: float, out_dtype):
     return out
 
 
-def moe_route_scores(x, wr, top_k: int, scoring: str = "softmax", renorm: bool = True):
+def moe_route_scores(x, wr, top_k: int, scoring: str = "softmax", renorm: bool = True, bias=None):
     """Router with f32 logits -> (topk_ids [T, k] int32, topk_w [T, k] f32); scoring "softmax" |
-    "sigmoid", `renorm`: divide the chosen scores by their sum."""
+    "sigmoid", `renorm`: divide the chosen scores by their sum ("softmax" + renorm = the softmax
+    over the chosen logits alone); `bias` [E] f32 is added to the logits."""
     if not _gpu(x):
-        return ref.moe_route_scores(x, wr, top_k, scoring, renorm)
+        return ref.moe_route_scores(x, wr, top_k, scoring, renorm, bias)
     T = x.shape[0]
     # logits: a GEMM with f32 accumulation and f32 output (steps of a few rows: one wave per
     # (token, expert) instead of a one-workgroup GEMM), then one wave per token picks
@@ -869,15 +877,18 @@ def moe_route_scores(x, wr, top_k: int, scoring: str = "softmax", renorm: bool =
         logits = linear_act(x, wr, out_dtype=torch.float32)
     ids = _empty(T, top_k, dtype=torch.int32, device=x.device)
     w = _empty(T, top_k, dtype=torch.float32, device=x.device)
-    torch.ops.bfly.moe_topk_scores(logits, top_k, {"softmax": 0, "sigmoid": 1}[scoring], bool(renorm), ids, w)
+    torch.ops.bfly.moe_topk_scores(logits, bias, top_k, {"softmax": 0, "sigmoid": 1}[scoring], bool(renorm), ids, w)
     return ids, w
 
 
-def moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit: float, alpha: float):
-    """Routed experts with a clamped GLU, each run on (routing score * x); see
-    ops.reference.moe_glu_ffn. gate_up_w [E, 2F, H], down_w [E, H, F]."""
+def moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit: float, alpha: float, up_offset: float = 1.0,
+                scale_input: bool = True):
+    """Routed GLU experts y = g' sigmoid(alpha g') (u' + up_offset) with g', u' clamped at `limit`
+    (inf, alpha 1, up_offset 0: the plain silu GLU). scale_input: each expert runs on (routing
+    score * x) and the outputs are summed; otherwise it runs on x and the sum is weighted by the
+    scores. See ops.reference.moe_glu_ffn. gate_up_w [E, 2F, H], down_w [E, H, F]."""
     if not _gpu(x):
-        return ref.moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit, alpha)
+        return ref.moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit, alpha, None, up_offset, scale_input)
     T, H = x.shape
     E, F = gate_up_w.shape[0], down_w.shape[2]
     TK = T * topk_ids.shape[1]
@@ -887,5 +898,112 @@ def moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit: float, alpha: flo
     hmid = _arena.get(dev, "moe_glu_mid", TK * F, x.dtype)
     y = _arena.get(dev, "moe_glu_y", TK * H, torch.float32)
     out = _empty(T, H, dtype=x.dtype, device=dev)
-    torch.ops.bfly.moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, float(limit), float(alpha), work, hmid, y, out)
+    torch.ops.bfly.moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, float(limit), float(alpha), float(up_offset),
+                               bool(scale_input), work, hmid, y, out)
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+# Post-norm residual stacks with latent attention (csrc/kernels/postnorm.hip)
+# ---------------------------------------------------------------------------------------
+def new_empty(*shape, dtype, device) -> torch.Tensor:
+    """A step's scratch tensor (poisoned under BFLY_POISON_OUTPUTS like every op output)."""
+    return _empty(*shape, dtype=dtype, device=device)
+
+
+def embed_scaled(ids, table, scale: float, out=None):
+    """out[t] = table[ids[t]] * scale, f32 [T, W]."""
+    if not _gpu(table):
+        return ref.embed_scaled(ids, table, scale, out)
+    if out is None:
+        out = _empty(ids.numel(), table.shape[1], dtype=torch.float32, device=table.device)
+    torch.ops.bfly.embed_scaled(ids, table, float(scale), out)
+    return out
+
+
+def conv_mix(x, w, state, state_slots, row_cu, positions, out_dtype):
+    """h_t = x_t + sum_j w[:, j] x_(t - taps + 1 + j): a causal per-channel convolution over the
+    rows of each sequence of a packed step, added to its input. x [T, W] f32; w [W, taps] f32 (None:
+    h = x); inputs before a sequence's first row of the step come from state[slot] ([slots,
+    taps - 1, W] f32, oldest first) and are zero before position 0. Returns h in out_dtype. The
+    state is not changed (conv_state_update_ does that, after every reader of the old state)."""
+    if not _gpu(x):
+        if w is None:
+            return x.to(out_dtype)
+        return ref.conv_mix(x, w, state, state_slots, row_cu, positions, out_dtype)
+    out = _empty(x.shape[0], x.shape[1], dtype=out_dtype, device=x.device)
+    torch.ops.bfly.conv_mix(x, w, state, state_slots, row_cu, positions, out)
+    return out
+
+
+def conv_state_update_(x, state, state_slots, row_cu, positions):
+    """state[slot] <- the last taps - 1 inputs of every sequence of the step (older ones shift)."""
+    if not _gpu(x):
+        return ref.conv_state_update_(x, state, state_slots, row_cu, positions)
+    torch.ops.bfly.conv_state_update(x, state, state_slots, row_cu, positions)
+    return state
+
+
+def post_norm_add(x, y, norm_w, norm_b, eps: float, scale, out, cast_dtype=None):
+    """out = x + scale * layer_norm(y) with weight and bias, all f32 (out may be x); returns out
+    rounded to cast_dtype (the next sublayer's GEMM operand), or None."""
+    if not _gpu(x):
+        return ref.post_norm_add(x, y, norm_w, norm_b, eps, scale, out, cast_dtype)
+    cast = None if cast_dtype is None else _empty(x.shape[0], x.shape[1], dtype=cast_dtype, device=x.device)
+    torch.ops.bfly.post_norm_add(x, y, norm_w, norm_b, float(eps), scale, out, cast)
+    return cast
+
+
+def post_norm_add_avg(x, y, norm_w, norm_b, eps: float, scale, stack, index: int, avg_w):
+    """X = x + scale * layer_norm(y) (y None: X = x); stack[index] = X; x <- sum_(j <= index)
+    avg_w[j] stack[j]: the residual update fused with a learned average over the results of all
+    layers so far. stack [n, T, W] f32, avg_w [index + 1] f32."""
+    if not _gpu(x):
+        return ref.post_norm_add_avg(x, y, norm_w, norm_b, eps, scale, stack, index, avg_w)
+    torch.ops.bfly.post_norm_add_avg(x, y, norm_w, norm_b, float(eps), scale, stack, int(index), avg_w)
+    return x
+
+
+def latent_prep(z, q_rank: int, kv_rank: int, rot_dim: int, heads: int, qn_w, kvn_w, eps: float, positions, inv_freq,
+                slots, k_cache, v_cache, out_dtype):
+    """Rows of z = [query latent | key/value latent | shared rotated key part | gate logits] ->
+    (RMS-normed query latent [T, q_rank], sigmoid gates [T, heads] f32); the normed key/value
+    latent and the rotated key part are appended to the paged caches K [blocks, 1, BS, kv_rank +
+    rot_dim], V [blocks, 1, kv_rank, BS]."""
+    if not _gpu(z):
+        return ref.latent_prep(z, q_rank, kv_rank, rot_dim, heads, qn_w, kvn_w, eps, positions, inv_freq, slots,
+                               k_cache, v_cache, out_dtype)
+    T = z.shape[0]
+    cq = _empty(T, q_rank, dtype=out_dtype, device=z.device)
+    gate = _empty(T, heads, dtype=torch.float32, device=z.device)
+    torch.ops.bfly.latent_prep(z, int(q_rank), int(kv_rank), int(rot_dim), int(heads), qn_w, kvn_w, float(eps), positions,
+                               inv_freq, slots, k_cache, v_cache, cq, gate)
+    return cq, gate
+
+
+def linear_heads(x, w, out):
+    """out[t, h] = w[h] x[t, h]: one small GEMM per head in a single launch. x [T, H, K] and out
+    [T, H, N] may be views into wider rows; w [H, N, K] contiguous."""
+    if not _gpu(x):
+        return ref.linear_heads(x, w, out)
+    torch.ops.bfly.linear_heads(x, w, out)
+    return out
+
+
+def rope_heads_copy(src, dst, positions, inv_freq):
+    """dst[t, h] = src[t, h] with the interleaved pairs (2i, 2i + 1), i < len(inv_freq), rotated by
+    positions[t] * inv_freq[i]; src, dst [T, H, n] views into wider rows."""
+    if not _gpu(src):
+        return ref.rope_heads_copy(src, dst, positions, inv_freq)
+    torch.ops.bfly.rope_heads_copy(src, dst, positions, inv_freq)
+    return dst
+
+
+def layer_norm_rows(x, w, b, eps: float, idx, out_dtype):
+    """Layer norm with weight and bias of rows idx (None: all) of the f32 residual x."""
+    if not _gpu(x):
+        return ref.layer_norm_rows(x, w, b, eps, idx, out_dtype)
+    R = x.shape[0] if idx is None else idx.numel()
+    out = _empty(R, x.shape[1], dtype=out_dtype, device=x.device)
+    torch.ops.bfly.layer_norm_rows(x, w, b, float(eps), idx, out)
     return out

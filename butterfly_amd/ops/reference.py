@@ -542,13 +542,21 @@ def ep_combine(back, slot):
 # MoE with clamped GLU experts. Caches of these mixers: K [blocks, G, BS, D], V [blocks, G, Dv, BS]
 # (V transposed), recurrent state [slots, H, D, Dv] f32.
 # ---------------------------------------------------------------------------------------
-def linear_act(x, w, bias=None, act="none", out_dtype=None):
-    """y = act(x w^T + bias), f32 accumulation; act: none | relu2 (relu squared)."""
+def xielu(y, a_pos: float, a_neg: float):
+    """z > 0: a_pos z^2 + z / 2;  z <= 0: a_neg (exp(z) - 1 - z) + z / 2."""
+    return torch.where(y > 0, a_pos * y * y + 0.5 * y, a_neg * (torch.expm1(y) - y) + 0.5 * y)
+
+
+def linear_act(x, w, bias=None, act="none", out_dtype=None, act_params=None):
+    """y = act(x w^T + bias), f32 accumulation; act: none | relu2 (relu squared) | xielu (the two
+    coefficients in act_params)."""
     y = x.float() @ w.float().t()
     if bias is not None:
         y = y + bias.float()
     if act == "relu2":
         y = torch.relu(y).square()
+    elif act == "xielu":
+        y = xielu(y, float(act_params[0]), float(act_params[1]))
     elif act != "none":
         raise ValueError(act)
     return y.to(out_dtype or x.dtype)
@@ -601,10 +609,12 @@ def rope_partial_kv(q, k, v, positions, inv_freq, slots, k_cache, v_cache):
     return q
 
 
-def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, window, keep_first, sink, out=None):
+def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, window, keep_first, sink, out=None,
+                      out_scale=None):
     """Row r of sequence s (rows row_cu[s] .. row_cu[s+1]) at position p attends to the cached
     keys j <= p of tables[s] with p - j < window or j < keep_first; the softmax denominator
-    also holds exp(sink[h])."""
+    also holds exp(sink[h]) (sink None: an ordinary softmax). out_scale [T, H] f32: every head's
+    output is multiplied by its entry (an output gate)."""
     T, H, D = q.shape
     G, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
     o = torch.zeros(T, H, Dv, dtype=torch.float32, device=q.device)
@@ -626,9 +636,14 @@ def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale, win
             g = h // (H // G)
             sc = (qs[:, h] @ K[g].t()) * scale
             sc = sc.masked_fill(~ok, float("-inf"))
-            sk = sink[h].float().expand(sc.shape[0], 1)
-            w = torch.softmax(torch.cat([sc, sk], 1), -1)[:, :-1]
+            if sink is None:
+                w = torch.softmax(sc, -1)
+            else:
+                sk = sink[h].float().expand(sc.shape[0], 1)
+                w = torch.softmax(torch.cat([sc, sk], 1), -1)[:, :-1]
             o[cu[s]:cu[s + 1], h] = w @ V[g]
+    if out_scale is not None:
+        o = o * out_scale.float()[:, :, None]
     o = o.to(q.dtype)
     if out is None:
         return o
@@ -666,10 +681,13 @@ def gla_out(o, g, norm_w, eps, out_dtype):
     return (y.reshape(T, H * Dv) * F.silu(g.float())).to(out_dtype)
 
 
-def moe_route_scores(x, wr, top_k, scoring="softmax", renorm=True):
+def moe_route_scores(x, wr, top_k, scoring="softmax", renorm=True, bias=None):
     """Router in f32. scoring "softmax" | "sigmoid"; the top_k largest scores are chosen (ties:
-    lowest expert id); `renorm`: the chosen scores are divided by their sum."""
+    lowest expert id); `renorm`: the chosen scores are divided by their sum (with "softmax" that
+    is the softmax over the chosen logits alone). `bias` [E] f32 is added to the logits."""
     logits = x.float() @ wr.float().t()
+    if bias is not None:
+        logits = logits + bias.float()
     sc = torch.softmax(logits, -1) if scoring == "softmax" else torch.sigmoid(logits)
     w, ids = torch.topk(sc, top_k, -1)
     if renorm:
@@ -677,11 +695,13 @@ def moe_route_scores(x, wr, top_k, scoring="softmax", renorm=True):
     return ids.to(torch.int32), w.contiguous()
 
 
-def moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit, alpha, out_dtype=None):
-    """Routed experts with clamped GLU: for every chosen (token, expert) the expert runs on
-    w * x: g = min(Wg h, limit), u = clamp(Wu h, -limit, limit), y = g sigmoid(alpha g) (u + 1),
-    output Wd y; a token's expert outputs are summed (f32). gate_up_w [E, 2F, H] (gate rows, then
-    up rows), down_w [E, H, F]."""
+def moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit, alpha, out_dtype=None, up_offset=1.0,
+                scale_input=True):
+    """Routed GLU experts: g = min(Wg h, limit), u = clamp(Wu h, -limit, limit),
+    y = g sigmoid(alpha g) (u + up_offset), output Wd y (limit inf, alpha 1, up_offset 0: the plain
+    silu GLU). scale_input: the expert runs on h = w * x and a token's expert outputs are summed;
+    otherwise it runs on x and the sum is weighted by w (f32). gate_up_w [E, 2F, H] (gate rows,
+    then up rows), down_w [E, H, F]."""
     T, H = x.shape
     Fd = down_w.shape[2]
     out = torch.zeros(T, H, dtype=torch.float32, device=x.device)
@@ -690,10 +710,145 @@ def moe_glu_ffn(x, topk_ids, topk_w, gate_up_w, down_w, limit, alpha, out_dtype=
             if e < 0:
                 continue
             tok = (topk_ids[:, j] == e).nonzero().flatten()
-            h = (x[tok].float() * topk_w[tok, j:j + 1].float()).to(x.dtype).float()
+            wj = topk_w[tok, j:j + 1].float()
+            h = (x[tok].float() * wj).to(x.dtype).float() if scale_input else x[tok].float()
             gu = h @ gate_up_w[e].float().t()
             g = gu[:, :Fd].clamp(max=limit)
             u = gu[:, Fd:].clamp(-limit, limit)
-            y = (g * torch.sigmoid(alpha * g) * (u + 1)).to(x.dtype).float()
-            out[tok] += y @ down_w[e].float().t()
+            y = (g * torch.sigmoid(alpha * g) * (u + up_offset)).to(x.dtype).float()
+            yd = y @ down_w[e].float().t()
+            out[tok] += yd if scale_input else wj * yd
     return out.to(out_dtype or x.dtype)
+
+
+# ---------------------------------------------------------------------------------------
+# Post-norm residual stacks with latent attention: scaled embedding, causal per-channel
+# convolution on a mixer's input (its last taps - 1 inputs pooled per sequence), layer norm on a
+# sublayer's output with a per-channel scale before the residual sum, a learned average over the
+# outputs of all earlier layers, latents / shared rotated key for an attention that caches only
+# those, per-head batched projections.
+# ---------------------------------------------------------------------------------------
+def embed_scaled(ids, table, scale, out=None):
+    """out[t] = table[ids[t]] * scale in f32."""
+    x = table[ids.long()].float() * scale
+    if out is None:
+        return x
+    out.copy_(x)
+    return out
+
+
+def conv_mix(x, w, state, state_slots, row_cu, positions, out_dtype):
+    """h_t = x_t + sum_j w[:, j] x_(t - taps + 1 + j) per channel, over time inside a sequence.
+    x [T, W] f32 packed rows; w [W, taps] f32; inputs before the step's first row of a sequence
+    come from state[slot] ([taps - 1, W] f32, oldest first) and are zero before position 0."""
+    T, W = x.shape
+    taps = w.shape[1]
+    h = x.clone()
+    cu, pos, sl = row_cu.tolist(), positions.tolist(), state_slots.tolist()
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if b <= a or sl[s] < 0:
+            continue
+        p0 = pos[a]
+        hist = state[sl[s]].clone() if taps > 1 else x.new_zeros(0, W)
+        for d in range(1, taps):           # hist[taps - 1 - d] is the input d steps before row a
+            if p0 - d < 0:
+                hist[taps - 1 - d] = 0
+        ext = torch.cat([hist, x[a:b]], 0)
+        for j in range(taps):
+            h[a:b] += w[:, j].float() * ext[j:j + (b - a)]
+    return h.to(out_dtype)
+
+
+def conv_state_update_(x, state, state_slots, row_cu, positions):
+    """After a step: state[slot] holds the sequence's last taps - 1 inputs (oldest first)."""
+    n = state.shape[1]
+    if n == 0:
+        return state
+    cu, pos, sl = row_cu.tolist(), positions.tolist(), state_slots.tolist()
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if b <= a or sl[s] < 0:
+            continue
+        old = state[sl[s]].clone()
+        for d in range(1, n + 1):
+            if pos[a] - d < 0:
+                old[n - d] = 0
+        state[sl[s]] = torch.cat([old, x[a:b]], 0)[-n:]
+    return state
+
+
+def _layer_norm_f32(y, w, b, eps):
+    y = y.float()
+    m = y.mean(-1, keepdim=True)
+    v = (y - m).pow(2).mean(-1, keepdim=True)
+    return (y - m) * torch.rsqrt(v + eps) * w.float() + b.float()
+
+
+def post_norm_add(x, y, norm_w, norm_b, eps, scale, out, cast_dtype=None):
+    """out = x + scale * layer_norm(y) (f32; out may be x); returns out rounded to cast_dtype
+    (None: nothing)."""
+    out.copy_(x + scale.float() * _layer_norm_f32(y, norm_w, norm_b, eps))
+    return None if cast_dtype is None else out.to(cast_dtype)
+
+
+def post_norm_add_avg(x, y, norm_w, norm_b, eps, scale, stack, index, avg_w):
+    """X = x + scale * layer_norm(y) (y None: X = x); stack[index] = X; x <- sum_j avg_w[j]
+    stack[j], j <= index. stack [n, T, W] f32, avg_w [index + 1] f32."""
+    X = x if y is None else x + scale.float() * _layer_norm_f32(y, norm_w, norm_b, eps)
+    stack[index] = X
+    x.copy_(torch.einsum("j,jtw->tw", avg_w.float(), stack[:index + 1]))
+    return x
+
+
+def latent_prep(z, q_rank, kv_rank, rot_dim, heads, qn_w, kvn_w, eps, positions, inv_freq, slots, k_cache, v_cache,
+                out_dtype):
+    """z [T, >= q_rank + kv_rank + rot_dim + heads] holds per row [query latent | key/value latent
+    | shared rotated key part | gate logits]. Returns (RMS-normed query latent [T, q_rank]
+    out_dtype, sigmoid(gate logits) [T, heads] f32) and appends [normed latent | rotated key part]
+    to K [blocks, 1, BS, kv_rank + rot_dim] and the normed latent to V [blocks, 1, kv_rank, BS]."""
+    zf = z.float()
+    o1, o2, o3 = q_rank, q_rank + kv_rank, q_rank + kv_rank + rot_dim
+    rms = lambda u, w: u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w.float()  # noqa: E731
+    cq = rms(zf[:, :o1], qn_w).to(out_dtype)
+    c = rms(zf[:, o1:o2], kvn_w)
+    kr = zf[:, o2:o3]
+    n = inv_freq.numel()
+    if n:
+        a = positions.float()[:, None] * inv_freq.float()[None]
+        cs, sn = torch.cos(a), torch.sin(a)
+        u, w = kr[:, 0:2 * n:2], kr[:, 1:2 * n:2]
+        kr = torch.cat([torch.stack([u * cs - w * sn, w * cs + u * sn], -1).flatten(-2), kr[:, 2 * n:]], 1)
+    gate = torch.sigmoid(zf[:, o3:o3 + heads]).contiguous()
+    bs = k_cache.shape[2]
+    ok = slots >= 0
+    sl = slots[ok].long()
+    k_cache[sl // bs, 0, sl % bs] = torch.cat([c, kr], 1)[ok].to(k_cache.dtype)
+    v_cache[sl // bs, 0, :, sl % bs] = c[ok].to(v_cache.dtype)
+    return cq, gate
+
+
+def linear_heads(x, w, out):
+    """out[t, h] = w[h] x[t, h] for every head: x [T, H, K] (a view), w [H, N, K], out [T, H, N]
+    (a view), f32 accumulation."""
+    out.copy_(torch.einsum("thk,hnk->thn", x.float(), w.float()).to(out.dtype))
+    return out
+
+
+def rope_heads_copy(src, dst, positions, inv_freq):
+    """dst[t, h] = src[t, h] with pairs (2i, 2i + 1), i < len(inv_freq), rotated by
+    positions[t] * inv_freq[i] (f32); src, dst [T, H, n] views."""
+    n = inv_freq.numel()
+    a = positions.float()[:, None] * inv_freq.float()[None]
+    c, s = torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
+    sf = src.float()
+    u, w = sf[..., 0:2 * n:2], sf[..., 1:2 * n:2]
+    r = torch.cat([torch.stack([u * c - w * s, w * c + u * s], -1).flatten(-2), sf[..., 2 * n:]], -1)
+    dst.copy_(r.to(dst.dtype))
+    return dst
+
+
+def layer_norm_rows(x, w, b, eps, idx, out_dtype):
+    """Layer norm (weight and bias, f32) of rows idx of x (None: all rows)."""
+    xs = x if idx is None else x[idx.long()]
+    return _layer_norm_f32(xs, w, b, eps).to(out_dtype)
