@@ -75,6 +75,10 @@ class ZinesunLM(PackedStack):
                               ffn=max(cfg.intermediate_size, 1), ffn0=0, vocab=vpad, vocab0=0, vocab_padded=vpad,
                               experts=max(cfg.num_experts, 1), expert0=0)
         self.cache_index = {sp["index"]: n for n, sp in enumerate(self.specs)}
+        # cached row widths: [latent | rotated key part] and the latent, padded with zeros to sizes
+        # the attention's matrix-core form tiles
+        self.cache_dims = [(ops.attn_window_pad(sp["kv_rank"] + sp["rot_dim"], dtype),
+                            ops.attn_window_pad(sp["kv_rank"], dtype)) for sp in self.specs]
         self.has_state = self.taps > 1            # the convolution's history
         self.state: list = []                     # set by allocate_state (the cache object owns the pool)
         self.layer_probe = None                   # debug hook: f(layer, residual [T, W] f32) after every layer
@@ -218,6 +222,10 @@ class ZinesunLM(PackedStack):
     # ------------------------------------------------------------------------------------
     # caches
     # ------------------------------------------------------------------------------------
+    def kv_bytes_per_token(self, dtype: Optional[torch.dtype] = None) -> int:
+        es = torch.empty((), dtype=dtype or self.dtype).element_size()
+        return max(1, sum(dk + dv for dk, dv in self.cache_dims) * es)
+
     def state_bytes_per_slot(self) -> int:
         return 4 * max(self.taps - 1, 0) * self.cfg.hidden_size * len(self.specs)
 
@@ -228,9 +236,9 @@ class ZinesunLM(PackedStack):
         dt = dtype or self.dtype
         if dt != self.dtype:
             raise NotImplementedError("Zinesun caches hold the model's element type")
-        return [(torch.zeros(num_blocks, 1, block_size, sp["kv_rank"] + sp["rot_dim"], dtype=dt, device=self.device),
-                 torch.zeros(num_blocks, 1, sp["kv_rank"], block_size, dtype=dt, device=self.device))
-                for sp in self.specs]
+        return [(torch.zeros(num_blocks, 1, block_size, dk, dtype=dt, device=self.device),
+                 torch.zeros(num_blocks, 1, dv, block_size, dtype=dt, device=self.device))
+                for dk, dv in self.cache_dims]
 
     def allocate_state(self, num_slots: int) -> list:
         """The convolution history pool: one [slots, taps - 1, W] f32 tensor per layer (a sequence's
@@ -301,13 +309,13 @@ class ZinesunLM(PackedStack):
                                    fb.positions, p[pre + "inv_freq"], fb.slots, kc, vc, self.dtype)
         q = ops.linear_act(cq, p[pre + "uq"])[:, :H * (D + rd)].view(T, H, D + rd)
         # queries in the latent space: [W_uk^T q_nope | rotated q_rot] per head
-        ql = ops.new_empty(T, H, R + rd, dtype=self.dtype, device=self.device)
+        ql = ops.new_empty(T, H, kc.shape[3], dtype=self.dtype, device=self.device)
         ops.linear_heads(q[:, :, :D], p[pre + "ukT"], ql[:, :, :R])
-        ops.rope_heads_copy(q[:, :, D:], ql[:, :, R:], fb.positions, p[pre + "inv_freq"])
+        ops.rope_heads_copy(q[:, :, D:], ql[:, :, R:], fb.positions, p[pre + "inv_freq"])    # (zero-fills the padding)
         ol = ops.attn_window_paged(ql, kc, vc, meta["tables"], meta["row_cu"], fb.positions, sp["scale"], sp["window"],
                                    0, None, row_map=meta["row_map"], fold_heads=True, out_scale=gate)
         o = ops.new_empty(T, H, Dv, dtype=self.dtype, device=self.device)
-        ops.linear_heads(ol, p[pre + "uv"], o)
+        ops.linear_heads(ol[:, :, :R], p[pre + "uv"], o)
         return ops.linear_act(o.view(T, H * Dv), p[pre + "o"])
 
     def _ffn(self, sp, pre, h):

@@ -990,9 +990,22 @@ def linear_heads(x, w, out):
     return out
 
 
+ATTN_MFMA_SIZES = (32, 64, 96, 128, 192, 256)
+
+
+def attn_window_pad(size: int, dtype) -> int:
+    """Head size a cache of `dtype` should be laid out with so that attn_window_paged takes its
+    matrix-core form (bf16: the next of ATTN_MFMA_SIZES; the padding holds zeros). Other types,
+    and sizes past the largest, stay as they are (the generic kernel takes any size)."""
+    if dtype != torch.bfloat16:
+        return size
+    return next((s for s in ATTN_MFMA_SIZES if s >= size), size)
+
+
 def rope_heads_copy(src, dst, positions, inv_freq):
-    """dst[t, h] = src[t, h] with the interleaved pairs (2i, 2i + 1), i < len(inv_freq), rotated by
-    positions[t] * inv_freq[i]; src, dst [T, H, n] views into wider rows."""
+    """dst[t, h, :n] = src[t, h] with the interleaved pairs (2i, 2i + 1), i < len(inv_freq), rotated
+    by positions[t] * inv_freq[i]; dst[t, h, n:] = 0. src [T, H, n], dst [T, H, >= n] views into
+    wider rows."""
     if not _gpu(src):
         return ref.rope_heads_copy(src, dst, positions, inv_freq)
     torch.ops.bfly.rope_heads_copy(src, dst, positions, inv_freq)

@@ -836,15 +836,16 @@ def linear_heads(x, w, out):
 
 
 def rope_heads_copy(src, dst, positions, inv_freq):
-    """dst[t, h] = src[t, h] with pairs (2i, 2i + 1), i < len(inv_freq), rotated by
-    positions[t] * inv_freq[i] (f32); src, dst [T, H, n] views."""
+    """dst[t, h, :n] = src[t, h] with pairs (2i, 2i + 1), i < len(inv_freq), rotated by
+    positions[t] * inv_freq[i] (f32); src [T, H, n], dst [T, H, >= n] views (the tail is zeroed)."""
     n = inv_freq.numel()
     a = positions.float()[:, None] * inv_freq.float()[None]
     c, s = torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
     sf = src.float()
     u, w = sf[..., 0:2 * n:2], sf[..., 1:2 * n:2]
     r = torch.cat([torch.stack([u * c - w * s, w * c + u * s], -1).flatten(-2), sf[..., 2 * n:]], -1)
-    dst.copy_(r.to(dst.dtype))
+    dst[..., :src.shape[-1]] = r.to(dst.dtype)
+    dst[..., src.shape[-1]:] = 0
     return dst
 
 

@@ -28,13 +28,14 @@ inline bool is_f32(const Tensor& t) {
 #define CHK_HEADS(t) \
   TORCH_CHECK((t).dim() == 3 && (t).stride(2) == 1 && (t).stride(1) == (t).size(2), #t " must be [T, heads, dim] rows")
 
-void gemm_any(const Tensor& x, const Tensor& w, const optional<Tensor>& bias, int64_t act, Tensor& out) {
+void gemm_any(const Tensor& x, const Tensor& w, const optional<Tensor>& bias, int64_t act, double a0, double a1,
+              Tensor& out) {
   CHK_GPU(x); CHK_GPU(w); CHK_GPU(out); CHK_SAME(x, w);
   TORCH_CHECK(x.dim() == 2 && w.dim() == 2 && out.dim() == 2, "gemm_any: 2-D operands");
   TORCH_CHECK(x.stride(1) == 1 && w.stride(1) == 1 && out.stride(1) == 1, "gemm_any: unit inner strides");
   const int64_t M = x.size(0), K = x.size(1), N = w.size(0);
   TORCH_CHECK(w.size(1) == K && out.size(0) == M && out.size(1) == N, "gemm_any: shapes");
-  TORCH_CHECK(act == 0 || act == 1, "gemm_any: act");
+  TORCH_CHECK(act >= 0 && act <= 2, "gemm_any: act");
   const bool f32 = is_f32(x);
   const bool of32 = out.scalar_type() == at::kFloat;
   TORCH_CHECK(of32 || out.scalar_type() == x.scalar_type(), "gemm_any: out type");
@@ -45,13 +46,26 @@ void gemm_any(const Tensor& x, const Tensor& w, const optional<Tensor>& bias, in
     b = bias->data_ptr();
   }
   bfly::launch_gemm_any(x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), b, out.data_ptr(), out.stride(0), (int)M,
-                        (int)N, (int)K, (int)act, f32, of32 && !f32, cur_stream());
+                        (int)N, (int)K, (int)act, (float)a0, (float)a1, f32, of32 && !f32, cur_stream());
 }
 
-void relu2_(Tensor& x) {
+// out[t, h] = w[h] x[t, h]: x [T, H, K], out [T, H, N] (views into wider rows), w [H, N, K]
+void linear_heads(const Tensor& x, const Tensor& w, Tensor& out) {
+  CHK_GPU(x); CHK_GPU(w); CHK_GPU(out); CHK_SAME(x, w); CHK_SAME(x, out);
+  TORCH_CHECK(x.dim() == 3 && w.dim() == 3 && out.dim() == 3 && w.is_contiguous() && x.stride(2) == 1 &&
+                  out.stride(2) == 1, "linear_heads: x [T, H, K], w [H, N, K], out [T, H, N]");
+  const int64_t T = x.size(0), H = x.size(1), K = x.size(2), N = w.size(1);
+  TORCH_CHECK(w.size(0) == H && w.size(2) == K && out.size(0) == T && out.size(1) == H && out.size(2) == N &&
+                  H <= 65535, "linear_heads: shapes");
+  bfly::launch_gemm_any(x.data_ptr(), x.stride(0), w.data_ptr(), K, nullptr, out.data_ptr(), out.stride(0), (int)T,
+                        (int)N, (int)K, 0, 0.f, 0.f, is_f32(x), false, cur_stream(), (int)H, x.stride(1), N * K,
+                        out.stride(1));
+}
+
+void act_(Tensor& x, int64_t act, double a0, double a1) {
   CHK_GPU(x);
-  TORCH_CHECK(x.is_contiguous(), "relu2_: contiguous");
-  bfly::launch_relu2(x.data_ptr(), x.numel(), is_f32(x), cur_stream());
+  TORCH_CHECK(x.is_contiguous() && act >= 0 && act <= 2, "act_: contiguous, act 0..2");
+  bfly::launch_act(x.data_ptr(), x.numel(), (int)act, (float)a0, (float)a1, is_f32(x), cur_stream());
 }
 
 void embed_norm_streams(const Tensor& ids, const Tensor& table, const Tensor& norm_w, double eps, double offset,
@@ -157,9 +171,10 @@ void row_seq(const Tensor& row_cu, Tensor& out) {
 
 void attn_window_paged(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, const Tensor& tables,
                        const Tensor& row_seq_t, const Tensor& row_cu, const Tensor& positions, double scale,
-                       int64_t window, int64_t keep_first, const Tensor& sink, Tensor& out) {
+                       int64_t window, int64_t keep_first, const optional<Tensor>& sink,
+                       const optional<Tensor>& out_scale, bool fold_heads, Tensor& out) {
   CHK_GPU(q); CHK_HEADS(q); CHK_SAME(k_cache, q); CHK_SAME(v_cache, q); CHK_SAME(out, q);
-  CHK_I32(tables); CHK_I32(row_seq_t); CHK_I32(positions); CHK_F32(sink);
+  CHK_I32(tables); CHK_I32(row_seq_t); CHK_I32(positions);
   const int64_t T = q.size(0), H = q.size(1), D = q.size(2);
   TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.is_contiguous(),
               "attn_window_paged: caches");
@@ -168,22 +183,34 @@ void attn_window_paged(const Tensor& q, const Tensor& k_cache, const Tensor& v_c
               "attn_window_paged: cache shapes K [blocks, G, BS, D], V [blocks, G, Dv, BS]");
   CHK_I32(row_cu);
   TORCH_CHECK(row_cu.numel() == tables.size(0) + 1, "attn_window_paged: row_cu");
-  TORCH_CHECK(G > 0 && H % G == 0 && Dv <= 256 && D <= 4096, "attn_window_paged: head counts / sizes");
-  TORCH_CHECK(tables.dim() == 2 && row_seq_t.numel() == T && positions.numel() == T && sink.numel() == H,
-              "attn_window_paged: index shapes");
+  TORCH_CHECK(G > 0 && H % G == 0 && Dv <= 512 && D <= 4096, "attn_window_paged: head counts / sizes");
+  TORCH_CHECK(tables.dim() == 2 && row_seq_t.numel() == T && positions.numel() == T, "attn_window_paged: index shapes");
+  const float *sinkp = nullptr, *gatep = nullptr;
+  if (sink.has_value()) {
+    CHK_F32(*sink);
+    TORCH_CHECK(sink->numel() == H, "attn_window_paged: sink [H]");
+    sinkp = sink->data_ptr<float>();
+  }
+  if (out_scale.has_value()) {
+    CHK_F32(*out_scale);
+    TORCH_CHECK(out_scale->numel() == T * H, "attn_window_paged: out_scale [T, H]");
+    gatep = out_scale->data_ptr<float>();
+  }
+  TORCH_CHECK(!fold_heads || G == 1, "attn_window_paged: fold_heads needs one shared key / value head");
   TORCH_CHECK(out.is_contiguous() && out.dim() == 3 && out.size(0) == T && out.size(1) == H && out.size(2) == Dv,
               "attn_window_paged: out");
   TORCH_CHECK(window >= 1 && keep_first >= 0, "attn_window_paged: window >= 1, keep_first >= 0");
   if (!is_f32(q) && bfly::launch_attn_window_mfma(q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                                   tables.data_ptr<int>(), (int)tables.size(1), row_cu.data_ptr<int>(),
                                                   (int)tables.size(0), positions.data_ptr<int>(), (float)scale,
-                                                  (int)window, (int)keep_first, sink.data_ptr<float>(), out.data_ptr(),
-                                                  (int)T, (int)H, (int)G, (int)D, (int)Dv, (int)bs, cur_stream()))
+                                                  (int)window, (int)keep_first, sinkp, gatep, out.data_ptr(),
+                                                  (int)T, (int)H, (int)G, (int)D, (int)Dv, (int)bs, fold_heads,
+                                                  cur_stream()))
     return;
   bfly::launch_attn_window_paged(q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                  tables.data_ptr<int>(), (int)tables.size(1), row_seq_t.data_ptr<int>(),
                                  (int)tables.size(0), positions.data_ptr<int>(), (float)scale, (int)window,
-                                 (int)keep_first, sink.data_ptr<float>(), out.data_ptr(), (int)T, (int)H, (int)G, (int)D,
+                                 (int)keep_first, sinkp, gatep, out.data_ptr(), (int)T, (int)H, (int)G, (int)D,
                                  (int)Dv, (int)bs, is_f32(q), cur_stream());
 }
 
@@ -226,13 +253,20 @@ void router_logits(const Tensor& x, const Tensor& wr, Tensor& logits) {
                              is_f32(x), cur_stream());
 }
 
-void moe_topk_scores(const Tensor& logits, int64_t top_k, int64_t scoring, bool renorm, Tensor& ids, Tensor& w) {
+void moe_topk_scores(const Tensor& logits, const optional<Tensor>& bias, int64_t top_k, int64_t scoring, bool renorm,
+                     Tensor& ids, Tensor& w) {
   CHK_GPU(logits); CHK_F32(logits); CHK_I32(ids); CHK_F32(w);
+  const float* bp = nullptr;
+  if (bias.has_value()) {
+    CHK_F32(*bias);
+    TORCH_CHECK(bias->numel() == logits.size(1), "moe_topk_scores: bias [E]");
+    bp = bias->data_ptr<float>();
+  }
   TORCH_CHECK(logits.dim() == 2, "moe_topk_scores: logits [T, E]");
   const int64_t T = logits.size(0), E = logits.size(1);
   TORCH_CHECK(E >= 1 && E <= 1024 && top_k >= 1 && top_k <= E, "moe_topk_scores: experts / top_k");
   TORCH_CHECK(ids.numel() == T * top_k && w.numel() == T * top_k, "moe_topk_scores: outputs");
-  bfly::launch_moe_topk_scores(logits.data_ptr<float>(), (int)top_k, (int)scoring, renorm, ids.data_ptr<int>(),
+  bfly::launch_moe_topk_scores(logits.data_ptr<float>(), bp, (int)top_k, (int)scoring, renorm, ids.data_ptr<int>(),
                                w.data_ptr<float>(), (int)T, (int)E, cur_stream());
 }
 
@@ -240,8 +274,8 @@ int64_t moe_sort_max_tiles(int64_t TK, int64_t E) { return bfly::moe_sort_max_ti
 
 // work: int32 [TK + (E + 1) + 2 * max_tiles + 1] = perm | offsets | tiles | ntiles
 void moe_glu_ffn(const Tensor& x, const Tensor& topk_ids, const Tensor& topk_w, const Tensor& gate_up_w,
-                 const Tensor& down_w, double limit, double alpha, Tensor& work, Tensor& hmid, Tensor& y,
-                 Tensor& out) {
+                 const Tensor& down_w, double limit, double alpha, double up_offset, bool scale_input, Tensor& work,
+                 Tensor& hmid, Tensor& y, Tensor& out) {
   CHK_GPU(x); CHK_SAME(x, gate_up_w); CHK_SAME(x, down_w); CHK_SAME(x, hmid); CHK_SAME(x, out);
   CHK_I32(topk_ids); CHK_F32(topk_w); CHK_I32(work); CHK_F32(y);
   TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1 && gate_up_w.dim() == 3 && down_w.dim() == 3 &&
@@ -264,12 +298,14 @@ void moe_glu_ffn(const Tensor& x, const Tensor& topk_ids, const Tensor& topk_w, 
   const bool f32 = is_f32(x);
   const int tr = bfly::moe_tile_rows((int)TK, (int)E, f32);
   bfly::launch_moe_sort(topk_ids.data_ptr<int>(), (int)TK, (int)E, perm, offsets, tiles, ntiles, tr, s);
-  bfly::launch_moe_glu_up(x.data_ptr(), x.stride(0), topk_w.data_ptr<float>(), (int)K, perm, offsets, tiles, ntiles,
-                          (int)mt, gate_up_w.data_ptr(), (float)limit, (float)alpha, hmid.data_ptr(), (int)Hd, (int)F,
-                          f32, tr, s);
+  // scores on the expert's input (the row is scaled and the outputs are summed) or on its output
+  bfly::launch_moe_glu_up(x.data_ptr(), x.stride(0), scale_input ? topk_w.data_ptr<float>() : nullptr, (int)K, perm,
+                          offsets, tiles, ntiles, (int)mt, gate_up_w.data_ptr(), (float)limit, (float)alpha,
+                          (float)up_offset, hmid.data_ptr(), (int)Hd, (int)F, f32, tr, s);
   bfly::launch_moe_down(hmid.data_ptr(), perm, offsets, tiles, ntiles, (int)mt, down_w.data_ptr(), y.data_ptr<float>(),
                         (int)Hd, (int)F, f32, tr, s);
-  bfly::launch_moe_sum(y.data_ptr<float>(), (int)K, out.data_ptr(), (int)T, (int)Hd, f32, s);
+  bfly::launch_moe_sum(y.data_ptr<float>(), scale_input ? nullptr : topk_w.data_ptr<float>(), (int)K, out.data_ptr(),
+                       (int)T, (int)Hd, f32, s);
 }
 
 void sample_greedy_f32(const Tensor& logits, int64_t vstart, Tensor& out_ids, Tensor& out_scores, bool check_finite) {
@@ -285,8 +321,9 @@ void sample_greedy_f32(const Tensor& logits, int64_t vstart, Tensor& out_ids, Te
 
 TORCH_LIBRARY_FRAGMENT(bfly, m) {
   m.def("sample_greedy_f32(Tensor logits, int vstart, Tensor(a!) out_ids, Tensor(b!) out_scores, bool check_finite) -> ()");
-  m.def("gemm_any(Tensor x, Tensor w, Tensor? bias, int act, Tensor(a!) out) -> ()");
-  m.def("relu2_(Tensor(a!) x) -> ()");
+  m.def("gemm_any(Tensor x, Tensor w, Tensor? bias, int act, float a0, float a1, Tensor(a!) out) -> ()");
+  m.def("linear_heads(Tensor x, Tensor w, Tensor(a!) out) -> ()");
+  m.def("act_(Tensor(a!) x, int act, float a0, float a1) -> ()");
   m.def("embed_norm_streams(Tensor ids, Tensor table, Tensor norm_w, float eps, float offset, Tensor(a!) xs) -> ()");
   m.def("hc_pre(Tensor xs, Tensor w_in, Tensor norm_w, float eps, float offset, Tensor(a!) out) -> ()");
   m.def("hc_post(Tensor(a!) xs, Tensor y, Tensor mix, Tensor w_out) -> ()");
@@ -297,21 +334,25 @@ TORCH_LIBRARY_FRAGMENT(bfly, m) {
         "Tensor(c!)? k_cache, Tensor(d!)? v_cache) -> ()");
   m.def("row_seq(Tensor row_cu, Tensor(a!) out) -> ()");
   m.def("attn_window_paged(Tensor q, Tensor k_cache, Tensor v_cache, Tensor tables, Tensor row_seq, Tensor row_cu, "
-        "Tensor positions, float scale, int window, int keep_first, Tensor sink, Tensor(a!) out) -> ()");
+        "Tensor positions, float scale, int window, int keep_first, Tensor? sink, Tensor? out_scale, bool fold_heads, "
+        "Tensor(a!) out) -> ()");
   m.def("gla_scan(Tensor q, Tensor k, Tensor v, Tensor z, Tensor(a!) state, Tensor state_slots, Tensor row_cu, "
         "Tensor positions, float tau, float q_scale, Tensor(b!) o) -> ()");
   m.def("gla_out(Tensor o, Tensor g, Tensor norm_w, float eps, Tensor(a!) out) -> ()");
   m.def("router_logits(Tensor x, Tensor wr, Tensor(a!) logits) -> ()");
-  m.def("moe_topk_scores(Tensor logits, int top_k, int scoring, bool renorm, Tensor(a!) ids, Tensor(b!) w) -> ()");
+  m.def("moe_topk_scores(Tensor logits, Tensor? bias, int top_k, int scoring, bool renorm, Tensor(a!) ids, "
+        "Tensor(b!) w) -> ()");
   m.def("moe_sort_max_tiles(int tk, int experts) -> int", &moe_sort_max_tiles);
   m.def("moe_glu_ffn(Tensor x, Tensor topk_ids, Tensor topk_w, Tensor gate_up_w, Tensor down_w, float limit, "
-        "float alpha, Tensor(a!) work, Tensor(b!) hmid, Tensor(c!) y, Tensor(d!) out) -> ()");
+        "float alpha, float up_offset, bool scale_input, Tensor(a!) work, Tensor(b!) hmid, Tensor(c!) y, "
+        "Tensor(d!) out) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(bfly, CUDA, m) {
   m.impl("sample_greedy_f32", &sample_greedy_f32);
   m.impl("gemm_any", &gemm_any);
-  m.impl("relu2_", &relu2_);
+  m.impl("linear_heads", &linear_heads);
+  m.impl("act_", &act_);
   m.impl("embed_norm_streams", &embed_norm_streams);
   m.impl("hc_pre", &hc_pre);
   m.impl("hc_post", &hc_post);

@@ -11,13 +11,17 @@
 
 namespace bfly {
 
-enum AnyAct { ACT_NONE = 0, ACT_RELU2 = 1 };
+enum AnyAct { ACT_NONE = 0, ACT_RELU2 = 1, ACT_XIELU = 2 };
 
-// out[M, N] = act(x[M, K] w[N, K]^T + bias[N]); `out_f32`: out is float whatever the inputs.
+// out[M, N] = act(x[M, K] w[N, K]^T + bias[N]); `out_f32`: out is float whatever the inputs. act:
+// squared ReLU, or xIELU with coefficients (a0, a1): v > 0: a0 v^2 + v / 2, else a1 (exp(v) - 1 - v) + v / 2.
+// batch > 1: `batch` independent problems (one per head, say) whose x / w / out start bx / bw / bo
+// elements apart, in one launch.
 void launch_gemm_any(const void* x, long ldx, const void* w, long ldw, const void* bias, void* out, long ldo,
-                     int M, int N, int K, int act, bool f32, bool out_f32, hipStream_t s);
-// x <- relu(x)^2 elementwise (n elements)
-void launch_relu2(void* x, long n, bool f32, hipStream_t s);
+                     int M, int N, int K, int act, float a0, float a1, bool f32, bool out_f32, hipStream_t s,
+                     int batch = 1, long bx = 0, long bw = 0, long bo = 0);
+// x <- act(x) elementwise (n elements)
+void launch_act(void* x, long n, int act, float a0, float a1, bool f32, hipStream_t s);
 
 // xs[t, s, :] = rms(table[ids[t]]) * (w + offset) for every stream s; xs f32 [T, S, W]
 void launch_embed_norm_streams(const int* ids, const void* table, const float* norm_w, float eps, float offset,
@@ -44,19 +48,21 @@ void launch_rope_partial_kv(void* q, long q_ld, void* k, long k_ld, const void* 
 // row_seq[t] = the sequence whose row range [row_cu[s], row_cu[s+1]) holds row t, else -1
 void launch_row_seq(const int* row_cu, int nseq, int* row_seq, int T, hipStream_t s);
 // Row t of sequence row_seq[t] (-1: padding row, output zero) at position p sees cached keys
-// j <= p with p - j < window or j < keep_first; the softmax denominator includes exp(sink[h]).
-// out [T, H, Dv] contiguous. Dv <= 256.
+// j <= p with p - j < window or j < keep_first; the softmax denominator includes exp(sink[h])
+// (sink == nullptr: an ordinary softmax); out_scale (nullable) [T, H] multiplies each head's output.
+// out [T, H, Dv] contiguous. Dv <= 512.
 void launch_attn_window_paged(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
                               int max_blocks, const int* row_seq, int nseq, const int* positions, float scale,
-                              int window, int keep_first, const float* sink, void* out, int T, int H, int G, int D,
-                              int Dv, int block_size, bool f32, hipStream_t s);
+                              int window, int keep_first, const float* sink, const float* out_scale, void* out, int T,
+                              int H, int G, int D, int Dv, int block_size, bool f32, hipStream_t s);
 
-// The MFMA form of launch_attn_window_paged over row_cu (bf16, 32-token pages, D in {32, 64, 128,
-// 256}, Dv in {32, 64, 128, 256}, 16-byte aligned q rows): false if the shape has no such form.
+// The MFMA form of launch_attn_window_paged over row_cu (bf16, 32-token pages, D and Dv in {32, 64,
+// 96, 128, 192, 256}, 16-byte aligned q rows): false if the shape has no such form. `fold` (G == 1):
+// tiles run over (token, head) pairs, so a token's heads share the pages they read.
 bool launch_attn_window_mfma(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
                              int max_blocks, const int* row_cu, int nseq, const int* positions, float scale, int window,
-                             int keep_first, const float* sink, void* out, int T, int H, int G, int D, int Dv,
-                             int block_size, hipStream_t s);
+                             int keep_first, const float* sink, const float* out_scale, void* out, int T, int H, int G,
+                             int D, int Dv, int block_size, bool fold, hipStream_t s);
 
 // Gated linear attention scan over packed rows (see ops.gla_scan). Returns < 0 if D > 256.
 int launch_gla_scan(const void* q, long q_ld, const void* k, long k_ld, const void* v, long v_ld, const void* z,
@@ -70,10 +76,10 @@ void launch_gla_out(const float* o, const void* g, long g_ld, const float* norm_
 // logits[t, e] = x[t] . wr[e] in f32, one wave per pair (for steps of a few rows)
 void launch_router_logits(const void* x, long ldx, const void* wr, float* logits, int T, int E, int Hd, bool f32,
                           hipStream_t s);
-// Router choice from f32 logits [T, E]: scoring 0 softmax / 1 sigmoid, top-k (ties: lowest id),
-// optional renorm. E <= 1024.
-void launch_moe_topk_scores(const float* logits, int top_k, int scoring, bool renorm, int* ids, float* w, int T, int E,
-                            hipStream_t s);
+// Router choice from f32 logits [T, E] (+ bias [E], nullable): scoring 0 softmax / 1 sigmoid, top-k
+// (ties: lowest id), optional renorm. E <= 1024.
+void launch_moe_topk_scores(const float* logits, const float* bias, int top_k, int scoring, bool renorm, int* ids,
+                            float* w, int T, int E, hipStream_t s);
 // Group the T*K (token, choice) pairs by expert: perm [TK] pair indices grouped by expert,
 // offsets [E + 1], tiles [max_tiles][2] = (expert, first row) of every tile_rows-row tile, ntiles [1].
 void launch_moe_sort(const int* ids, int TK, int E, int* perm, int* offsets, int* tiles, int* ntiles, int tile_rows,
@@ -81,14 +87,15 @@ void launch_moe_sort(const int* ids, int TK, int E, int* perm, int* offsets, int
 int moe_sort_max_tiles(int TK, int E);
 // rows per tile of the grouped expert GEMMs for this problem (64, or 128 for large bf16 groups)
 int moe_tile_rows(int TK, int E, bool f32);
-// hmid[r, f] = glu(gate, up) of expert e(r) on (w x) for grouped row r
+// hmid[r, f] = g' sigmoid(alpha g') (u' + up_offset), (g', u') the clamped gate / up products of
+// expert e(r) on (w x) for grouped row r (topk_w == nullptr: on x itself)
 void launch_moe_glu_up(const void* x, long ldx, const float* topk_w, int K, const int* perm, const int* offsets,
                        const int* tiles, const int* ntiles, int max_tiles, const void* gate_up_w, float limit,
-                       float alpha, void* hmid, int Hd, int F, bool f32, int tile_rows, hipStream_t s);
+                       float alpha, float up_offset, void* hmid, int Hd, int F, bool f32, int tile_rows, hipStream_t s);
 // y[perm[r], :] = down_e(r) hmid[r]     (y f32, pair order)
 void launch_moe_down(const void* hmid, const int* perm, const int* offsets, const int* tiles, const int* ntiles,
                      int max_tiles, const void* down_w, float* y, int Hd, int F, bool f32, int tile_rows, hipStream_t s);
-// out[t] = sum_j y[t * K + j]
-void launch_moe_sum(const float* y, int K, void* out, int T, int Hd, bool f32, hipStream_t s);
+// out[t] = sum_j wts[t * K + j] y[t * K + j]   (wts == nullptr: the plain sum)
+void launch_moe_sum(const float* y, const float* wts, int K, void* out, int T, int Hd, bool f32, hipStream_t s);
 
 }  // namespace bfly

@@ -23,6 +23,14 @@ constexpr int TM = 64, TN = 64, TK = 16, LDP = TM + 4;
 template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)*p; }
 template <typename T> __device__ __forceinline__ T cvt(float v) { return (T)v; }
 
+// epilogue activations: squared ReLU; xIELU with coefficients (a0, a1): v > 0: a0 v^2 + v / 2,
+// else a1 (exp(v) - 1 - v) + v / 2
+__device__ __forceinline__ float apply_act(float v, int act, float a0, float a1) {
+  if (act == ACT_RELU2) { v = fmaxf(v, 0.f); return v * v; }
+  if (act == ACT_XIELU) return v > 0.f ? fmaf(a0 * v, v, 0.5f * v) : fmaf(a1, expm1f(v) - v, 0.5f * v);
+  return v;
+}
+
 // acc[i][j] += sum_k A(row0 + ty*4 + i, k) * B(col0 + tx*4 + j, k); la(r, k) / lb(c, k) return
 // the operand element as float (0 outside the problem).
 template <typename LA, typename LB>
@@ -56,9 +64,13 @@ __device__ __forceinline__ void tile_mac(float (&acc)[4][4], LA la, LB lb, int K
 template <typename T, typename TO>
 __global__ __launch_bounds__(256) void gemm_any_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ w,
                                                        long ldw, const T* __restrict__ bias, TO* __restrict__ out,
-                                                       long ldo, int M, int N, int K, int act) {
+                                                       long ldo, int M, int N, int K, int act, float a0, float a1,
+                                                       long bx, long bw, long bo) {
   __shared__ float As[TK][LDP], Bs[TK][LDP];
   const int row0 = blockIdx.y * TM, col0 = blockIdx.x * TN;
+  x += blockIdx.z * bx;            // batched form: one problem per blockIdx.z (e.g. per head)
+  w += blockIdx.z * bw;
+  out += blockIdx.z * bo;
   float acc[4][4] = {};
   tile_mac(
       acc,
@@ -75,18 +87,15 @@ __global__ __launch_bounds__(256) void gemm_any_kernel(const T* __restrict__ x, 
       if (c >= N) continue;
       float v = acc[i][j];
       if (bias) v += ldf(bias + c);
-      if (act == ACT_RELU2) { v = fmaxf(v, 0.f); v = v * v; }
-      out[(long)r * ldo + c] = cvt<TO>(v);
+      out[(long)r * ldo + c] = cvt<TO>(apply_act(v, act, a0, a1));
     }
   }
 }
 
 template <typename T>
-__global__ void relu2_kernel(T* x, long n) {
-  for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
-    float v = fmaxf((float)x[i], 0.f);
-    x[i] = (T)(v * v);
-  }
+__global__ void act_kernel(T* x, long n, int act, float a0, float a1) {
+  for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+    x[i] = (T)apply_act((float)x[i], act, a0, a1);
 }
 
 // One workgroup. counts -> offsets -> placement (order inside an expert's group is arbitrary:
@@ -133,7 +142,7 @@ __global__ __launch_bounds__(256) void moe_glu_up_kernel(const T* __restrict__ x
                                                          const int* __restrict__ perm, const int* __restrict__ offsets_e,
                                                          const int* __restrict__ tiles, const int* __restrict__ ntiles,
                                                          const T* __restrict__ gu_w, float limit, float alpha,
-                                                         T* __restrict__ hmid, int Hd, int F) {
+                                                         float up_offset, T* __restrict__ hmid, int Hd, int F) {
   if ((int)blockIdx.y >= ntiles[0]) return;
   __shared__ float As[TK][LDP], Bs[TK][LDP];
   __shared__ int tok[TM];
@@ -145,7 +154,7 @@ __global__ __launch_bounds__(256) void moe_glu_up_kernel(const T* __restrict__ x
     const int r = r0 + threadIdx.x;
     int p = r < rend ? perm[r] : -1;
     tok[threadIdx.x] = p < 0 ? -1 : p / Kc;
-    wt[threadIdx.x] = p < 0 ? 0.f : topk_w[p];
+    wt[threadIdx.x] = p < 0 ? 0.f : (topk_w ? topk_w[p] : 1.f);      // no scores: the row as it is
   }
   __syncthreads();
   const T* wg = gu_w + (long)e * 2 * F * Hd;
@@ -171,7 +180,7 @@ __global__ __launch_bounds__(256) void moe_glu_up_kernel(const T* __restrict__ x
       if (c >= F) continue;
       const float gg = fminf(g[i][j], limit);
       const float uu = fminf(fmaxf(u[i][j], -limit), limit);
-      const float y = gg / (1.f + expf(-alpha * gg)) * (uu + 1.f);
+      const float y = gg / (1.f + expf(-alpha * gg)) * (uu + up_offset);
       hmid[(long)r * F + c] = cvt<T>(y);
     }
   }
@@ -208,13 +217,18 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ hmi
 }
 
 template <typename T>
-__global__ void moe_sum_kernel(const float* __restrict__ y, int Kc, T* __restrict__ out, long T_, int Hd) {
+__global__ void moe_sum_kernel(const float* __restrict__ y, const float* __restrict__ wts, int Kc, T* __restrict__ out,
+                               long T_, int Hd) {
   const long n = T_ * Hd;
   for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
     const long t = i / Hd;
     const int c = (int)(i % Hd);
     float s = 0.f;
-    for (int j = 0; j < Kc; ++j) s += y[(t * Kc + j) * Hd + c];
+    if (wts) {
+      for (int j = 0; j < Kc; ++j) s = fmaf(wts[t * Kc + j], y[(t * Kc + j) * Hd + c], s);
+    } else {
+      for (int j = 0; j < Kc; ++j) s += y[(t * Kc + j) * Hd + c];
+    }
     out[i] = (T)s;
   }
 }
@@ -237,12 +251,13 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const T* __restrict_
 
 // Router choice of one token per wave from its f32 logits [E]: softmax or sigmoid scores, K rounds
 // of arg-max over the experts (ties to the lowest id).
-__global__ __launch_bounds__(64) void moe_topk_scores_kernel(const float* __restrict__ logits, int top_k, int scoring,
+__global__ __launch_bounds__(64) void moe_topk_scores_kernel(const float* __restrict__ logits,
+                                                             const float* __restrict__ bias, int top_k, int scoring,
                                                              int renorm, int* __restrict__ ids, float* __restrict__ w,
                                                              int E) {
   __shared__ float sc[1024];
   const int t = blockIdx.x, lane = threadIdx.x;
-  for (int e = lane; e < E; e += 64) sc[e] = logits[(long)t * E + e];
+  for (int e = lane; e < E; e += 64) sc[e] = logits[(long)t * E + e] + (bias ? bias[e] : 0.f);
   __syncthreads();
   if (scoring == 0) {
     float mx = -INFINITY;
@@ -477,10 +492,14 @@ template <typename TO, int WT>
 __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(const bf16* __restrict__ x, long ldx,
                                                             const bf16* __restrict__ w, long ldw,
                                                             const bf16* __restrict__ bias, TO* __restrict__ out,
-                                                            long ldo, int M, int N, int K, int act) {
+                                                            long ldo, int M, int N, int K, int act, float a0, float a1,
+                                                            long bx, long bw, long bo) {
   constexpr int BT = 32 * WT;
   __shared__ __attribute__((aligned(16))) bf16 Xs[BT][MLD], Ws[BT][MLD];
   const int row0 = blockIdx.y * BT, col0 = blockIdx.x * BT;
+  x += blockIdx.z * bx;
+  w += blockIdx.z * bw;
+  out += blockIdx.z * bo;
   BFLY_ZERO_ACC(acc);
   tile_mac_mfma<WT>(
       acc, [&](int r) { return RowRef{row0 + r < M ? x + (long)(row0 + r) * ldx : nullptr, 1.f}; },
@@ -489,8 +508,7 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(const bf16* __restri
     const int r = row0 + m, c = col0 + n;
     if (r >= M || c >= N) return;
     if (bias) v += (float)bias[c];
-    if (act == ACT_RELU2) { v = fmaxf(v, 0.f); v = v * v; }
-    out[(long)r * ldo + c] = (TO)v;
+    out[(long)r * ldo + c] = (TO)apply_act(v, act, a0, a1);
   });
 }
 
@@ -503,7 +521,7 @@ __global__ __launch_bounds__(256) void moe_glu_up_mfma_kernel(const bf16* __rest
                                                               const int* __restrict__ tiles,
                                                               const int* __restrict__ ntiles,
                                                               const bf16* __restrict__ gu_w, float limit, float alpha,
-                                                              bf16* __restrict__ hmid, int Hd, int F) {
+                                                              float up_offset, bf16* __restrict__ hmid, int Hd, int F) {
   if ((int)blockIdx.y >= ntiles[0]) return;
   constexpr int BT = 32 * WT;
   // small groups (decode): gate and up share one K loop, so both panels' weight segments are in
@@ -518,7 +536,7 @@ __global__ __launch_bounds__(256) void moe_glu_up_mfma_kernel(const bf16* __rest
   // the expert's input row: the token row times its routing score, rounded to bf16
   auto rowX = [&](int r) {
     const int p = r0 + r < rend ? perm[r0 + r] : -1;
-    return p < 0 ? RowRef{nullptr, 1.f} : RowRef{x + (long)(p / Kc) * ldx, topk_w[p]};
+    return p < 0 ? RowRef{nullptr, 1.f} : RowRef{x + (long)(p / Kc) * ldx, topk_w ? topk_w[p] : 1.f};
   };
   BFLY_ZERO_ACC(g);
   BFLY_ZERO_ACC(u);
@@ -542,7 +560,7 @@ __global__ __launch_bounds__(256) void moe_glu_up_mfma_kernel(const bf16* __rest
         if (r >= rend || c >= F) continue;
         const float gg = fminf(g[tn][tm][i], limit);
         const float uu = fminf(fmaxf(u[tn][tm][i], -limit), limit);
-        hmid[(long)r * F + c] = (bf16)(gg / (1.f + expf(-alpha * gg)) * (uu + 1.f));
+        hmid[(long)r * F + c] = (bf16)(gg / (1.f + expf(-alpha * gg)) * (uu + up_offset));
       }
 }
 
@@ -575,34 +593,35 @@ inline int ew_blocks(long n) { return (int)std::min<long>(4096, std::max<long>(1
 }  // namespace
 
 void launch_gemm_any(const void* x, long ldx, const void* w, long ldw, const void* bias, void* out, long ldo,
-                     int M, int N, int K, int act, bool f32, bool out_f32, hipStream_t s) {
-  if (M <= 0 || N <= 0) return;
-  dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM);
+                     int M, int N, int K, int act, float a0, float a1, bool f32, bool out_f32, hipStream_t s,
+                     int batch, long bx, long bw, long bo) {
+  if (M <= 0 || N <= 0 || batch <= 0) return;
+  dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM, batch);
   if (!f32 && M >= 512 && N >= 128) {        // large row counts: the 128 x 128 workgroup tile
-    dim3 g2((N + 127) / 128, (M + 127) / 128);
+    dim3 g2((N + 127) / 128, (M + 127) / 128, batch);
     if (out_f32)
       gemm_any_mfma_kernel<float, 4><<<g2, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
-                                                        (float*)out, ldo, M, N, K, act);
+                                                        (float*)out, ldo, M, N, K, act, a0, a1, bx, bw, bo);
     else
       gemm_any_mfma_kernel<bf16, 4><<<g2, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
-                                                       (bf16*)out, ldo, M, N, K, act);
+                                                       (bf16*)out, ldo, M, N, K, act, a0, a1, bx, bw, bo);
     return;
   }
   if (f32)
     gemm_any_kernel<float, float><<<grid, 256, 0, s>>>((const float*)x, ldx, (const float*)w, ldw, (const float*)bias,
-                                                       (float*)out, ldo, M, N, K, act);
+                                                       (float*)out, ldo, M, N, K, act, a0, a1, bx, bw, bo);
   else if (out_f32)
     gemm_any_mfma_kernel<float, 2><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
-                                                     (float*)out, ldo, M, N, K, act);
+                                                     (float*)out, ldo, M, N, K, act, a0, a1, bx, bw, bo);
   else
     gemm_any_mfma_kernel<bf16, 2><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)w, ldw, (const bf16*)bias,
-                                                    (bf16*)out, ldo, M, N, K, act);
+                                                    (bf16*)out, ldo, M, N, K, act, a0, a1, bx, bw, bo);
 }
 
-void launch_relu2(void* x, long n, bool f32, hipStream_t s) {
-  if (n <= 0) return;
-  if (f32) relu2_kernel<float><<<ew_blocks(n), 256, 0, s>>>((float*)x, n);
-  else relu2_kernel<bf16><<<ew_blocks(n), 256, 0, s>>>((bf16*)x, n);
+void launch_act(void* x, long n, int act, float a0, float a1, bool f32, hipStream_t s) {
+  if (n <= 0 || act == ACT_NONE) return;
+  if (f32) act_kernel<float><<<ew_blocks(n), 256, 0, s>>>((float*)x, n, act, a0, a1);
+  else act_kernel<bf16><<<ew_blocks(n), 256, 0, s>>>((bf16*)x, n, act, a0, a1);
 }
 
 void launch_router_logits(const void* x, long ldx, const void* wr, float* logits, int T, int E, int Hd, bool f32,
@@ -613,10 +632,10 @@ void launch_router_logits(const void* x, long ldx, const void* wr, float* logits
   else router_logits_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)x, ldx, (const bf16*)wr, logits, E, Hd);
 }
 
-void launch_moe_topk_scores(const float* logits, int top_k, int scoring, bool renorm, int* ids, float* w, int T, int E,
-                            hipStream_t s) {
+void launch_moe_topk_scores(const float* logits, const float* bias, int top_k, int scoring, bool renorm, int* ids,
+                            float* w, int T, int E, hipStream_t s) {
   if (T <= 0) return;
-  moe_topk_scores_kernel<<<T, 64, 0, s>>>(logits, top_k, scoring, renorm, ids, w, E);
+  moe_topk_scores_kernel<<<T, 64, 0, s>>>(logits, bias, top_k, scoring, renorm, ids, w, E);
 }
 
 int moe_sort_max_tiles(int TKp, int E) { return (TKp + 63) / 64 + E; }
@@ -631,20 +650,20 @@ void launch_moe_sort(const int* ids, int TKp, int E, int* perm, int* offsets, in
 
 void launch_moe_glu_up(const void* x, long ldx, const float* topk_w, int K, const int* perm, const int* offsets,
                        const int* tiles, const int* ntiles, int max_tiles, const void* gate_up_w, float limit,
-                       float alpha, void* hmid, int Hd, int F, bool f32, int tile_rows, hipStream_t s) {
+                       float alpha, float up_offset, void* hmid, int Hd, int F, bool f32, int tile_rows, hipStream_t s) {
   if (tile_rows == 128) {
     dim3 g2((F + 127) / 128, max_tiles);
     moe_glu_up_mfma_kernel<4><<<g2, 256, 0, s>>>((const bf16*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
-                                                 (const bf16*)gate_up_w, limit, alpha, (bf16*)hmid, Hd, F);
+                                                 (const bf16*)gate_up_w, limit, alpha, up_offset, (bf16*)hmid, Hd, F);
     return;
   }
   dim3 grid((F + TN - 1) / TN, max_tiles);
   if (f32)
     moe_glu_up_kernel<float><<<grid, 256, 0, s>>>((const float*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
-                                                  (const float*)gate_up_w, limit, alpha, (float*)hmid, Hd, F);
+                                                  (const float*)gate_up_w, limit, alpha, up_offset, (float*)hmid, Hd, F);
   else
     moe_glu_up_mfma_kernel<2><<<grid, 256, 0, s>>>((const bf16*)x, ldx, topk_w, K, perm, offsets, tiles, ntiles,
-                                                (const bf16*)gate_up_w, limit, alpha, (bf16*)hmid, Hd, F);
+                                                (const bf16*)gate_up_w, limit, alpha, up_offset, (bf16*)hmid, Hd, F);
 }
 
 void launch_moe_down(const void* hmid, const int* perm, const int* offsets, const int* tiles, const int* ntiles,
@@ -664,11 +683,11 @@ void launch_moe_down(const void* hmid, const int* perm, const int* offsets, cons
                                               Hd, F);
 }
 
-void launch_moe_sum(const float* y, int K, void* out, int T, int Hd, bool f32, hipStream_t s) {
+void launch_moe_sum(const float* y, const float* wts, int K, void* out, int T, int Hd, bool f32, hipStream_t s) {
   const long n = (long)T * Hd;
   if (n <= 0) return;
-  if (f32) moe_sum_kernel<float><<<ew_blocks(n), 256, 0, s>>>(y, K, (float*)out, T, Hd);
-  else moe_sum_kernel<bf16><<<ew_blocks(n), 256, 0, s>>>(y, K, (bf16*)out, T, Hd);
+  if (f32) moe_sum_kernel<float><<<ew_blocks(n), 256, 0, s>>>(y, wts, K, (float*)out, T, Hd);
+  else moe_sum_kernel<bf16><<<ew_blocks(n), 256, 0, s>>>(y, wts, K, (bf16*)out, T, Hd);
 }
 
 }  // namespace bfly

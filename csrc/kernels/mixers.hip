@@ -62,8 +62,10 @@ __global__ __launch_bounds__(256) void rope_partial_kv_kernel(T* __restrict__ q,
 
 // One wave per (row, query head). Keys are visited 64 at a time (one per lane) with an online
 // softmax seeded by the sink: m = sink, l = 1, acc = 0, so the sink counts once in the
-// denominator and has no value. Lane `l` then owns output dims l, l + 64, ... (Dv <= 256).
-constexpr int kMaxDvLane = 4;
+// denominator and has no value (no sink: m very low, l = 0, an ordinary softmax). Lane `l` then
+// owns output dims l, l + 64, ... (Dv <= 512). out_scale (nullable) [T, H] multiplies the output
+// of every (row, head): an output gate.
+constexpr int kMaxDvLane = 8;
 
 template <typename T>
 __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restrict__ q, long q_ld,
@@ -73,8 +75,10 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
                                                                const int* __restrict__ row_seq,
                                                                const int* __restrict__ positions, float scale,
                                                                int window, int keep_first,
-                                                               const float* __restrict__ sink, T* __restrict__ out,
-                                                               int H, int G, int D, int Dv, int bs) {
+                                                               const float* __restrict__ sink,
+                                                               const float* __restrict__ out_scale,
+                                                               T* __restrict__ out, int H, int G, int D, int Dv,
+                                                               int bs) {
   extern __shared__ float smem[];      // q [D] | p [64] | key row base index [64] (as int)
   float* sq = smem;
   float* sp = smem + D;
@@ -94,8 +98,8 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
   const int lo = max(0, p - window + 1);
   const int n1 = min(keep_first, lo);          // kept first positions outside the window
   const int total = n1 + (p - lo + 1);
-  float m = sink[h], l = 1.f;
-  float acc[kMaxDvLane] = {0.f, 0.f, 0.f, 0.f};
+  float m = sink ? sink[h] : -1e30f, l = sink ? 1.f : 0.f;
+  float acc[kMaxDvLane] = {};
   for (int i0 = 0; i0 < total; i0 += 64) {
     const int i = i0 + lane;
     float sc = -INFINITY;
@@ -128,7 +132,7 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
       acc[c] = a;
     }
   }
-  const float inv = 1.f / l;
+  const float inv = (out_scale ? out_scale[t * H + h] : 1.f) / l;
 #pragma unroll
   for (int c = 0; c < kMaxDvLane; ++c) {
     const int d = lane + 64 * c;
@@ -146,7 +150,10 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
 // page's keys as the MFMA k index in the order the score tiles leave them (keys 4g..4g+3 and
 // 16+4g..16+4g+3 in lane group g), which the transposed V page serves with two 8-byte reads.
 // The next page's K and V fragments are loaded before the current page is multiplied. The sink
-// seeds wave 0's softmax (m = sink, l = 1). The per-element mask settles the window edges.
+// seeds wave 0's softmax (m = sink, l = 1; without a sink m is very low and l = 0). The
+// per-element mask settles the window edges. `fold` > 0 (one shared key / value head, G = 1,
+// fold = H): the tile's 16 rows run over (token, head) pairs, row r = token * H + head, so the
+// heads of a decoded token share one tile and a token's heads walk the cached pages once.
 template <int DS, int DVT>
 __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __restrict__ q, long q_ld,
                                                                const bf16* __restrict__ k_cache,
@@ -156,7 +163,8 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
                                                                const int* __restrict__ positions, float scale,
                                                                int window, int keep_first,
                                                                const float* __restrict__ sink,
-                                                               bf16* __restrict__ out, int H, int G) {
+                                                               const float* __restrict__ out_scale,
+                                                               bf16* __restrict__ out, int H, int G, int fold) {
   constexpr int D = 32 * DS, Dv = 16 * DVT, BS = 32;
   extern __shared__ float smem[];          // o of waves 1-3 [3][DVT][4][64] | m [3][16] | l [3][16]
   float* so = smem;
@@ -164,10 +172,10 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
   float* sl = sm + 48;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int tile = blockIdx.x;
-  const int h = blockIdx.y, g = h / (H / G);
+  const int rf = fold > 0 ? fold : 1;       // tile rows per token
   int s = 0, row0 = 0, rend = 0;
   for (; s < nseq; ++s) {
-    const int a = row_cu[s], b = row_cu[s + 1];
+    const int a = row_cu[s] * rf, b = row_cu[s + 1] * rf;
     const int nt = (b - a + 15) >> 4;
     if (tile < nt) { row0 = a + 16 * tile; rend = b; break; }
     tile -= nt;
@@ -175,7 +183,10 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
   if (s >= nseq) return;                   // (the whole workgroup: the tile is per workgroup)
   const int qr = lane & 15, gg = lane >> 4;
   const bool rv = row0 + qr < rend;
-  const long row = rv ? row0 + qr : row0;
+  const long frow = rv ? row0 + qr : row0;
+  const long row = frow / rf;                                   // the token's row
+  const int h = fold > 0 ? (int)(frow % rf) : (int)blockIdx.y;  // this lane's query head
+  const int g = fold > 0 ? 0 : h / (H / G);
   const int p = rv ? positions[row] : -1;
   int pmin = rv ? p : 0x7fffffff, pmax = p;
 #pragma unroll
@@ -188,7 +199,7 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
   for (int ds = 0; ds < DS; ++ds)
     qf[ds] = *reinterpret_cast<const bf16x8*>(q + row * q_ld + (long)h * D + 32 * ds + 8 * gg);
   const int* tab = tables + (long)s * max_blocks;
-  float m = wave == 0 ? sink[h] : -1e30f, l = wave == 0 ? 1.f : 0.f;
+  float m = (wave == 0 && sink) ? sink[h] : -1e30f, l = (wave == 0 && sink) ? 1.f : 0.f;
   f32x4 o[DVT];
 #pragma unroll
   for (int t = 0; t < DVT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -297,7 +308,7 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
       for (int i = 0; i < 4; ++i) o[t][i] = o[t][i] * c0 + po[(t * 4 + i) * 64 + lane] * cu;
   }
   if (!rv) return;
-  const float inv = 1.f / l;
+  const float inv = (out_scale ? out_scale[row * H + h] : 1.f) / l;
   bf16* orow = out + (row * H + h) * Dv;
 #pragma unroll
   for (int t = 0; t < DVT; ++t) {
@@ -465,16 +476,21 @@ void launch_row_seq(const int* row_cu, int nseq, int* row_seq, int T, hipStream_
 template <int DS>
 static bool attn_mfma_dv(const bf16* q, long q_ld, const bf16* kc, const bf16* vc, const int* tables, int max_blocks,
                          const int* row_cu, int nseq, const int* positions, float scale, int window, int keep_first,
-                         const float* sink, bf16* out, int T, int H, int G, int Dv, hipStream_t s) {
+                         const float* sink, const float* out_scale, bf16* out, int T, int H, int G, int Dv, bool fold,
+                         hipStream_t s) {
   // one workgroup per 16-row tile; every sequence adds at most one partly filled tile
-  dim3 grid((T + 15) / 16 + nseq, H);
+  dim3 grid(((fold ? T * H : T) + 15) / 16 + nseq, fold ? 1 : H);
+  const int fd = fold ? H : 0;
 #define BFLY_ATT(DVT)                                                                                          \
   attn_window_mfma_kernel<DS, DVT><<<grid, 256, (3 * DVT * 256 + 96) * sizeof(float), s>>>(                    \
-      q, q_ld, kc, vc, tables, max_blocks, row_cu, nseq, positions, scale, window, keep_first, sink, out, H, G)
+      q, q_ld, kc, vc, tables, max_blocks, row_cu, nseq, positions, scale, window, keep_first, sink, out_scale, out, H, \
+      G, fd)
   switch (Dv) {
     case 32: BFLY_ATT(2); return true;
     case 64: BFLY_ATT(4); return true;
+    case 96: BFLY_ATT(6); return true;
     case 128: BFLY_ATT(8); return true;
+    case 192: BFLY_ATT(12); return true;
     case 256: BFLY_ATT(16); return true;
     default: return false;
   }
@@ -483,17 +499,19 @@ static bool attn_mfma_dv(const bf16* q, long q_ld, const bf16* kc, const bf16* v
 
 bool launch_attn_window_mfma(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
                              int max_blocks, const int* row_cu, int nseq, const int* positions, float scale, int window,
-                             int keep_first, const float* sink, void* out, int T, int H, int G, int D, int Dv,
-                             int block_size, hipStream_t s) {
-  if (block_size != 32 || (q_ld & 7) || (reinterpret_cast<uintptr_t>(q) & 15)) return false;
+                             int keep_first, const float* sink, const float* out_scale, void* out, int T, int H, int G,
+                             int D, int Dv, int block_size, bool fold, hipStream_t s) {
+  if (block_size != 32 || (q_ld & 7) || (reinterpret_cast<uintptr_t>(q) & 15) || (fold && G != 1)) return false;
   if (T <= 0) return true;
 #define BFLY_ATTD(DS)                                                                                          \
   return attn_mfma_dv<DS>((const bf16*)q, q_ld, (const bf16*)k_cache, (const bf16*)v_cache, tables, max_blocks, row_cu, \
-                          nseq, positions, scale, window, keep_first, sink, (bf16*)out, T, H, G, Dv, s)
+                          nseq, positions, scale, window, keep_first, sink, out_scale, (bf16*)out, T, H, G, Dv, fold, s)
   switch (D) {
     case 32: BFLY_ATTD(1);
     case 64: BFLY_ATTD(2);
+    case 96: BFLY_ATTD(3);
     case 128: BFLY_ATTD(4);
+    case 192: BFLY_ATTD(6);
     case 256: BFLY_ATTD(8);
     default: return false;
   }
@@ -502,8 +520,8 @@ bool launch_attn_window_mfma(const void* q, long q_ld, const void* k_cache, cons
 
 void launch_attn_window_paged(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
                               int max_blocks, const int* row_seq, int nseq, const int* positions, float scale,
-                              int window, int keep_first, const float* sink, void* out, int T, int H, int G, int D,
-                              int Dv, int block_size, bool f32, hipStream_t s) {
+                              int window, int keep_first, const float* sink, const float* out_scale, void* out, int T,
+                              int H, int G, int D, int Dv, int block_size, bool f32, hipStream_t s) {
   if (T <= 0) return;
   (void)nseq;
   dim3 grid(T, H);
@@ -511,13 +529,13 @@ void launch_attn_window_paged(const void* q, long q_ld, const void* k_cache, con
   if (f32)
     attn_window_paged_kernel<float><<<grid, 64, sm, s>>>((const float*)q, q_ld, (const float*)k_cache,
                                                          (const float*)v_cache, tables, max_blocks, row_seq, positions,
-                                                         scale, window, keep_first, sink, (float*)out, H, G, D, Dv,
-                                                         block_size);
+                                                         scale, window, keep_first, sink, out_scale, (float*)out, H, G,
+                                                         D, Dv, block_size);
   else
     attn_window_paged_kernel<bf16><<<grid, 64, sm, s>>>((const bf16*)q, q_ld, (const bf16*)k_cache,
                                                         (const bf16*)v_cache, tables, max_blocks, row_seq, positions,
-                                                        scale, window, keep_first, sink, (bf16*)out, H, G, D, Dv,
-                                                        block_size);
+                                                        scale, window, keep_first, sink, out_scale, (bf16*)out, H, G, D,
+                                                        Dv, block_size);
 }
 
 template <typename T>
