@@ -235,12 +235,12 @@ def layer_spec(index: int, L: dict) -> dict:
         rot = m.get("rot") or {}
         mask = m.get("mask") or {"size": 1 << 30}
         sp.update(rot_dim=int(m.get("rot_dim", 0)), kv_rank=int(m["kv_rank"]), q_rank=int(m["q_rank"]),
-                  rot_base=float(rot.get("base", 10000.0)),
+                  rot_base=float(rot.get("base", 10000.0)), rot_dims=int(rot.get("dims", m.get("rot_dim", 0))),
                   scale=float(m.get("scale", (sp["dim"] + int(m.get("rot_dim", 0))) ** -0.5)),
                   window=int(mask["size"]))
-        if int(rot.get("dims", sp["rot_dim"])) != sp["rot_dim"]:
-            raise ValueError(f"layer {index}: the rotated part is rot_dim wide (rot.dims must equal it)")
-        if sp["window"] < 1 or sp["rot_dim"] % 2 or min(sp["kv_rank"], sp["q_rank"], sp["dim"] + sp["rot_dim"]) < 1:
+        if sp["rot_dims"] > sp["rot_dim"] or sp["rot_dims"] % 2:
+            raise ValueError(f"layer {index}: rot.dims must be even and at most rot_dim")
+        if sp["window"] < 1 or min(sp["kv_rank"], sp["q_rank"], sp["dim"] + sp["rot_dim"]) < 1:
             raise ValueError(f"layer {index}: bad latent-attention sizes")
     elif t == "gla":
         sp.update(tau=float(m["tau"]))

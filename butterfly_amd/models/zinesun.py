@@ -115,8 +115,9 @@ class ZinesunLM(PackedStack):
             p[pre + "ukT"] = z(H, R, D)               # W_uk per head, transposed: q_lat = ukT[h] q_nope
             p[pre + "uv"] = z(H, Dv, R)
             p[pre + "o"] = z(W, H * Dv)
-            i = torch.arange(rd // 2, dtype=torch.float64)
-            p[pre + "inv_freq"] = (sp["rot_base"] ** (-2.0 * i / max(rd, 1))).to(torch.float32).to(self.device)
+            # frequencies of the rotated pairs of the rot_dim part (its first rot_dims dimensions)
+            i = torch.arange(sp["rot_dims"] // 2, dtype=torch.float64)
+            p[pre + "inv_freq"] = (sp["rot_base"] ** (-2.0 * i / max(sp["rot_dims"], 1))).to(torch.float32).to(self.device)
             fs = sp["ffn"]
             if fs:
                 p[pre + "norm2"], p[pre + "norm2.b"], p[pre + "ls2"] = f(W), f(W), f(W)

@@ -744,13 +744,14 @@ def conv_mix(x, w, state, state_slots, row_cu, positions, out_dtype):
     T, W = x.shape
     taps = w.shape[1]
     h = x.clone()
-    cu, pos, sl = row_cu.tolist(), positions.tolist(), state_slots.tolist()
+    cu, pos = row_cu.tolist(), positions.tolist()
+    sl = state_slots.tolist() if state_slots is not None else [0] * (len(cu) - 1)
     for s in range(len(cu) - 1):
         a, b = cu[s], cu[s + 1]
-        if b <= a or sl[s] < 0:
+        if b <= a:
             continue
         p0 = pos[a]
-        hist = state[sl[s]].clone() if taps > 1 else x.new_zeros(0, W)
+        hist = state[sl[s]].clone() if (taps > 1 and sl[s] >= 0) else x.new_zeros(max(taps - 1, 0), W)
         for d in range(1, taps):           # hist[taps - 1 - d] is the input d steps before row a
             if p0 - d < 0:
                 hist[taps - 1 - d] = 0
