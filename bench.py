@@ -92,6 +92,9 @@ def build_parser() -> argparse.ArgumentParser:
                     help="single-stage layouts: host waits for each step's tokens before scheduling the "
                          "next (default: EngineConfig.async_decode, the next step overlaps the host work)")
     ap.add_argument("--out", default=None, help="also write the JSON line here")
+    ap.add_argument("--mixer-family", default="nesizen", choices=["nesizen", "zinesun"],
+                    help="with --mixer-compare: the heterogeneous family that is timed (nesizen: beside a Mixtral "
+                         "stack; zinesun: latent attention beside a Nesizen stack of plain windowed attention)")
     ap.add_argument("--mixer-compare", default=None, metavar="SIZES",
                     help="instead of the headline run: prefill and decode throughput of a Nesizen stack "
                          "(windowed attention, shared keys, gated linear attention, sigmoid MoE) beside a "
@@ -176,7 +179,27 @@ def run_mixer_compare(a) -> int:
         mix = ModelConfig(name=f"mixtral-{size}", arch="mixtral", vocab_size=32000, hidden_size=W,
                           intermediate_size=eff, num_layers=4, num_heads=H, num_kv_heads=G, head_dim=D,
                           max_position=32768, rope_theta=1e6, num_experts=E, experts_per_token=top, init_std=0.05)
-        for cfg in (nes, mix):
+        pair = (nes, mix)
+        if a.mixer_family == "zinesun":
+            # latent attention (cached rows 192 + 64 wide, queries through a rank-3W/4 latent, 128-wide
+            # heads) beside plain windowed GQA attention of the same heads, both with the same dense
+            # and routed feed-forwards, window and page size; one residual stream in the counterpart
+            lat = {"heads": H, "dim": D, "rot_dim": 64, "vdim": D, "kv_rank": 192, "q_rank": 3 * W // 4,
+                   "rot": {"dims": 64, "base": 1e6}, "scale": (D + 64) ** -0.5, "mask": {"size": win}}
+            zmoe = {"kind": "moe", "expert": {"ff": eff}, "router": {"experts": E, "top": top}}
+            dns = {"kind": "dense", "ff": dff}
+            zin = ModelConfig.from_zinesun({"architecture": "Zinesun", "vocab": 32000, "width": W,
+                                            "norm": {"eps": 1e-6}, "canon": {"taps": 4},
+                                            "embedding": {"scale": W ** 0.5}, "layers": [
+                                                {"type": "latent_attention", "mixer": lat, "mlp": f}
+                                                for f in (dns, zmoe, dns, zmoe)]}, name=f"zinesun-{size}")
+            plain = dict(attn, mask={"size": win, "keep_first": 0})
+            nes2 = ModelConfig.from_nesizen({"architecture": "Nesizen", "vocab": 32000, "width": W, "streams": 1,
+                                             "norm": {"eps": 1e-6}, "layers": [
+                                                 {"type": "attention", "mixer": plain, "mlp": f}
+                                                 for f in (dns, moe, dns, moe)]}, name=f"nesizen-attn-{size}")
+            pair = (zin, nes2)
+        for cfg in pair:
             ecfg = EngineConfig(max_batch=B, max_seq_len=P + K + Wm + 8, max_prefill_tokens=8192,
                                 kv_cache_tokens=B * (P + K + Wm + 40), use_graphs=not a.no_graphs,
                                 async_decode=False, prefix_caching=False,

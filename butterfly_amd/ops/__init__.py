@@ -838,8 +838,13 @@ def attn_window_paged(q, k_cache, v_cache, tables, row_cu, positions, scale: flo
         out = _empty(q.shape[0], q.shape[1], v_cache.shape[2], dtype=q.dtype, device=q.device)
     if row_map is None:
         row_map = row_seq(row_cu, q.shape[0])
+    # steps of few rows (decoding): scratch so that several workgroups can share a tile's pages
+    part = None
+    rows = q.shape[0] * q.shape[1]
+    if q.dtype == torch.bfloat16 and rows <= 2048:
+        part = _arena.get(q.device, "attn_window_part", 16 * rows * (v_cache.shape[2] + 2), torch.float32)
     torch.ops.bfly.attn_window_paged(q, k_cache, v_cache, tables, row_map, row_cu, positions, float(scale), int(window),
-                                     int(keep_first), sink, out_scale, bool(fold_heads), out)
+                                     int(keep_first), sink, out_scale, bool(fold_heads), part, out)
     return out
 
 

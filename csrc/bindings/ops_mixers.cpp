@@ -172,7 +172,7 @@ void row_seq(const Tensor& row_cu, Tensor& out) {
 void attn_window_paged(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, const Tensor& tables,
                        const Tensor& row_seq_t, const Tensor& row_cu, const Tensor& positions, double scale,
                        int64_t window, int64_t keep_first, const optional<Tensor>& sink,
-                       const optional<Tensor>& out_scale, bool fold_heads, Tensor& out) {
+                       const optional<Tensor>& out_scale, bool fold_heads, const optional<Tensor>& part, Tensor& out) {
   CHK_GPU(q); CHK_HEADS(q); CHK_SAME(k_cache, q); CHK_SAME(v_cache, q); CHK_SAME(out, q);
   CHK_I32(tables); CHK_I32(row_seq_t); CHK_I32(positions);
   const int64_t T = q.size(0), H = q.size(1), D = q.size(2);
@@ -197,6 +197,13 @@ void attn_window_paged(const Tensor& q, const Tensor& k_cache, const Tensor& v_c
     gatep = out_scale->data_ptr<float>();
   }
   TORCH_CHECK(!fold_heads || G == 1, "attn_window_paged: fold_heads needs one shared key / value head");
+  float* partp = nullptr;
+  int64_t part_n = 0;
+  if (part.has_value()) {
+    CHK_F32(*part);
+    partp = part->data_ptr<float>();
+    part_n = part->numel();
+  }
   TORCH_CHECK(out.is_contiguous() && out.dim() == 3 && out.size(0) == T && out.size(1) == H && out.size(2) == Dv,
               "attn_window_paged: out");
   TORCH_CHECK(window >= 1 && keep_first >= 0, "attn_window_paged: window >= 1, keep_first >= 0");
@@ -204,8 +211,8 @@ void attn_window_paged(const Tensor& q, const Tensor& k_cache, const Tensor& v_c
                                                   tables.data_ptr<int>(), (int)tables.size(1), row_cu.data_ptr<int>(),
                                                   (int)tables.size(0), positions.data_ptr<int>(), (float)scale,
                                                   (int)window, (int)keep_first, sinkp, gatep, out.data_ptr(),
-                                                  (int)T, (int)H, (int)G, (int)D, (int)Dv, (int)bs, fold_heads,
-                                                  cur_stream()))
+                                                  (int)T, (int)H, (int)G, (int)D, (int)Dv, (int)bs, fold_heads, partp,
+                                                  (long)part_n, cur_stream()))
     return;
   bfly::launch_attn_window_paged(q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                  tables.data_ptr<int>(), (int)tables.size(1), row_seq_t.data_ptr<int>(),
@@ -335,7 +342,7 @@ TORCH_LIBRARY_FRAGMENT(bfly, m) {
   m.def("row_seq(Tensor row_cu, Tensor(a!) out) -> ()");
   m.def("attn_window_paged(Tensor q, Tensor k_cache, Tensor v_cache, Tensor tables, Tensor row_seq, Tensor row_cu, "
         "Tensor positions, float scale, int window, int keep_first, Tensor? sink, Tensor? out_scale, bool fold_heads, "
-        "Tensor(a!) out) -> ()");
+        "Tensor(b!)? part, Tensor(a!) out) -> ()");
   m.def("gla_scan(Tensor q, Tensor k, Tensor v, Tensor z, Tensor(a!) state, Tensor state_slots, Tensor row_cu, "
         "Tensor positions, float tau, float q_scale, Tensor(b!) o) -> ()");
   m.def("gla_out(Tensor o, Tensor g, Tensor norm_w, float eps, Tensor(a!) out) -> ()");

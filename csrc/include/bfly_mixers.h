@@ -58,11 +58,13 @@ void launch_attn_window_paged(const void* q, long q_ld, const void* k_cache, con
 
 // The MFMA form of launch_attn_window_paged over row_cu (bf16, 32-token pages, D and Dv in {32, 64,
 // 96, 128, 192, 256}, 16-byte aligned q rows): false if the shape has no such form. `fold` (G == 1):
-// tiles run over (token, head) pairs, so a token's heads share the pages they read.
+// tiles run over (token, head) pairs, so a token's heads share the pages they read. `part` (nullable,
+// part_floats f32): scratch for steps of few tiles, whose pages are then split over several
+// workgroups per tile (T * H * (Dv + 2) floats per split).
 bool launch_attn_window_mfma(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
                              int max_blocks, const int* row_cu, int nseq, const int* positions, float scale, int window,
                              int keep_first, const float* sink, const float* out_scale, void* out, int T, int H, int G,
-                             int D, int Dv, int block_size, bool fold, hipStream_t s);
+                             int D, int Dv, int block_size, bool fold, float* part, long part_floats, hipStream_t s);
 
 // Gated linear attention scan over packed rows (see ops.gla_scan). Returns < 0 if D > 256.
 int launch_gla_scan(const void* q, long q_ld, const void* k, long k_ld, const void* v, long v_ld, const void* z,

@@ -154,6 +154,8 @@ __global__ __launch_bounds__(64) void attn_window_paged_kernel(const T* __restri
 // per-element mask settles the window edges. `fold` > 0 (one shared key / value head, G = 1,
 // fold = H): the tile's 16 rows run over (token, head) pairs, row r = token * H + head, so the
 // heads of a decoded token share one tile and a token's heads walk the cached pages once.
+// `nsplit` > 1 (steps of few tiles, i.e. decoding): gridDim.z workgroups share a tile's pages,
+// each leaves its unnormalised (o, m, l) per row in `part` and attn_split_merge_kernel folds them.
 template <int DS, int DVT>
 __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __restrict__ q, long q_ld,
                                                                const bf16* __restrict__ k_cache,
@@ -164,8 +166,11 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
                                                                int window, int keep_first,
                                                                const float* __restrict__ sink,
                                                                const float* __restrict__ out_scale,
-                                                               bf16* __restrict__ out, int H, int G, int fold) {
+                                                               bf16* __restrict__ out, int H, int G, int fold,
+                                                               int nsplit, float* __restrict__ part,
+                                                               long part_rows) {
   constexpr int D = 32 * DS, Dv = 16 * DVT, BS = 32;
+  const int split = blockIdx.z;
   extern __shared__ float smem[];          // o of waves 1-3 [3][DVT][4][64] | m [3][16] | l [3][16]
   float* so = smem;
   float* sm = smem + 3 * DVT * 256;
@@ -199,7 +204,8 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
   for (int ds = 0; ds < DS; ++ds)
     qf[ds] = *reinterpret_cast<const bf16x8*>(q + row * q_ld + (long)h * D + 32 * ds + 8 * gg);
   const int* tab = tables + (long)s * max_blocks;
-  float m = (wave == 0 && sink) ? sink[h] : -1e30f, l = (wave == 0 && sink) ? 1.f : 0.f;
+  const bool seeded = wave == 0 && split == 0 && sink;
+  float m = seeded ? sink[h] : -1e30f, l = seeded ? 1.f : 0.f;
   f32x4 o[DVT];
 #pragma unroll
   for (int t = 0; t < DVT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -225,11 +231,12 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
     }
   };
   bf16x8 kf[2][DS], vf[DVT];
-  int pi = wave;
+  const int pstep = 4 * nsplit;
+  int pi = wave + 4 * split;
   if (pi < npages) load_kv(page_of(pi), kf, vf);
   while (pi < npages) {
     const int pg = page_of(pi);
-    const int ni = pi + 4;
+    const int ni = pi + pstep;
     bf16x8 nkf[2][DS], nvf[DVT];
     if (ni < npages) load_kv(page_of(ni), nkf, nvf);
     f32x4 st[2];
@@ -308,6 +315,15 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
       for (int i = 0; i < 4; ++i) o[t][i] = o[t][i] * c0 + po[(t * 4 + i) * 64 + lane] * cu;
   }
   if (!rv) return;
+  if (nsplit > 1) {
+    float* pp = part + ((long)split * part_rows + (row * H + h)) * (Dv + 2);
+#pragma unroll
+    for (int t = 0; t < DVT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pp[16 * t + 4 * gg + i] = o[t][i];
+    if (gg == 0) { pp[Dv] = m; pp[Dv + 1] = l; }
+    return;
+  }
   const float inv = (out_scale ? out_scale[row * H + h] : 1.f) / l;
   bf16* orow = out + (row * H + h) * Dv;
 #pragma unroll
@@ -316,6 +332,30 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
 #pragma unroll
     for (int i = 0; i < 4; ++i) w[i] = (bf16)(o[t][i] * inv);
     *reinterpret_cast<bf16x4*>(orow + 16 * t + 4 * gg) = w;
+  }
+}
+
+// One wave per (row, head): fold the nsplit partial results part[split][row][o (Dv) | m | l].
+__global__ __launch_bounds__(64) void attn_split_merge_kernel(const float* __restrict__ part, long part_rows,
+                                                              int nsplit, const float* __restrict__ out_scale,
+                                                              bf16* __restrict__ out, int Dv) {
+  const long r = blockIdx.x;
+  const int lane = threadIdx.x;
+  float m = -1e30f;
+  for (int s = 0; s < nsplit; ++s) m = fmaxf(m, part[((long)s * part_rows + r) * (Dv + 2) + Dv]);
+  float l = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float* pp = part + ((long)s * part_rows + r) * (Dv + 2);
+    l += pp[Dv + 1] * __expf(pp[Dv] - m);
+  }
+  const float inv = (out_scale ? out_scale[r] : 1.f) / l;
+  for (int d = lane; d < Dv; d += 64) {
+    float a = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float* pp = part + ((long)s * part_rows + r) * (Dv + 2);
+      a += pp[d] * __expf(pp[Dv] - m);
+    }
+    out[r * Dv + d] = (bf16)(a * inv);
   }
 }
 
@@ -477,35 +517,49 @@ template <int DS>
 static bool attn_mfma_dv(const bf16* q, long q_ld, const bf16* kc, const bf16* vc, const int* tables, int max_blocks,
                          const int* row_cu, int nseq, const int* positions, float scale, int window, int keep_first,
                          const float* sink, const float* out_scale, bf16* out, int T, int H, int G, int Dv, bool fold,
-                         hipStream_t s) {
+                         int nsplit, float* part, hipStream_t s) {
   // one workgroup per 16-row tile; every sequence adds at most one partly filled tile
-  dim3 grid(((fold ? T * H : T) + 15) / 16 + nseq, fold ? 1 : H);
+  dim3 grid(((fold ? T * H : T) + 15) / 16 + nseq, fold ? 1 : H, nsplit);
   const int fd = fold ? H : 0;
+  const long prow = (long)T * H;
 #define BFLY_ATT(DVT)                                                                                          \
   attn_window_mfma_kernel<DS, DVT><<<grid, 256, (3 * DVT * 256 + 96) * sizeof(float), s>>>(                    \
       q, q_ld, kc, vc, tables, max_blocks, row_cu, nseq, positions, scale, window, keep_first, sink, out_scale, out, H, \
-      G, fd)
+      G, fd, nsplit, part, prow)
   switch (Dv) {
-    case 32: BFLY_ATT(2); return true;
-    case 64: BFLY_ATT(4); return true;
-    case 96: BFLY_ATT(6); return true;
-    case 128: BFLY_ATT(8); return true;
-    case 192: BFLY_ATT(12); return true;
-    case 256: BFLY_ATT(16); return true;
+    case 32: BFLY_ATT(2); break;
+    case 64: BFLY_ATT(4); break;
+    case 96: BFLY_ATT(6); break;
+    case 128: BFLY_ATT(8); break;
+    case 192: BFLY_ATT(12); break;
+    case 256: BFLY_ATT(16); break;
     default: return false;
   }
+  if (nsplit > 1) attn_split_merge_kernel<<<(unsigned)prow, 64, 0, s>>>(part, prow, nsplit, out_scale, out, Dv);
+  return true;
 #undef BFLY_ATT
 }
 
 bool launch_attn_window_mfma(const void* q, long q_ld, const void* k_cache, const void* v_cache, const int* tables,
                              int max_blocks, const int* row_cu, int nseq, const int* positions, float scale, int window,
                              int keep_first, const float* sink, const float* out_scale, void* out, int T, int H, int G,
-                             int D, int Dv, int block_size, bool fold, hipStream_t s) {
+                             int D, int Dv, int block_size, bool fold, float* part, long part_floats, hipStream_t s) {
   if (block_size != 32 || (q_ld & 7) || (reinterpret_cast<uintptr_t>(q) & 15) || (fold && G != 1)) return false;
   if (T <= 0) return true;
+  // few tiles (decoding): several workgroups share a tile's pages, as many as fill the chip, the
+  // pages of a row (window and table width bound them) and the scratch allow
+  int nsplit = 1;
+  {
+    const long tiles = (long)(((fold ? T * H : T) + 15) / 16 + nseq) * (fold ? 1 : H);
+    const long pages = std::min<long>((long)window / 32 + 2 + (keep_first + 31) / 32, max_blocks);
+    const long fit = part ? part_floats / ((long)T * H * (Dv + 2)) : 1;
+    nsplit = (int)std::max<long>(1, std::min<long>(std::min<long>((256 + tiles - 1) / tiles, pages / 8),
+                                                    std::min<long>(fit, 16)));
+  }
 #define BFLY_ATTD(DS)                                                                                          \
   return attn_mfma_dv<DS>((const bf16*)q, q_ld, (const bf16*)k_cache, (const bf16*)v_cache, tables, max_blocks, row_cu, \
-                          nseq, positions, scale, window, keep_first, sink, out_scale, (bf16*)out, T, H, G, Dv, fold, s)
+                          nseq, positions, scale, window, keep_first, sink, out_scale, (bf16*)out, T, H, G, Dv, fold,    \
+                          nsplit, part, s)
   switch (D) {
     case 32: BFLY_ATTD(1);
     case 64: BFLY_ATTD(2);

@@ -42,6 +42,7 @@ __device__ __forceinline__ int seq_of_row(const int* __restrict__ row_cu, int ns
   return (nseq > 0 && row_cu[lo] <= t && t < row_cu[lo + 1]) ? lo : -1;
 }
 
+// one thread per (row, channel): the taps' loads are independent of one another
 template <typename TO>
 __global__ __launch_bounds__(256) void conv_mix_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                        const float* __restrict__ state,
@@ -50,27 +51,27 @@ __global__ __launch_bounds__(256) void conv_mix_kernel(const float* __restrict__
                                                        const int* __restrict__ positions, TO* __restrict__ out,
                                                        int W, int taps) {
   const int t = blockIdx.x;
-  const float* xr = x + (long)t * W;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= W) return;
+  const float xc = x[(long)t * W + c];
   const int s = (w && taps > 0) ? seq_of_row(row_cu, nseq, t) : -1;
   if (s < 0) {                       // no convolution, or a row outside every sequence
-    for (int c = threadIdx.x; c < W; c += blockDim.x) out[(long)t * W + c] = (TO)xr[c];
+    out[(long)t * W + c] = (TO)xc;
     return;
   }
   const int a = row_cu[s], p = positions[t];
   const int slot = state_slots ? state_slots[s] : -1;
   const int n = taps - 1;
-  for (int c = threadIdx.x; c < W; c += blockDim.x) {
-    float h = xr[c];
-    for (int j = 0; j < taps; ++j) {
-      const int d = n - j;           // the input d steps back
-      float v = 0.f;
-      if (d == 0) v = xr[c];
-      else if (t - d >= a) v = x[(long)(t - d) * W + c];
-      else if (p - d >= 0 && slot >= 0) v = state[((long)slot * n + (n - (d - (t - a)))) * W + c];
-      h = fmaf(w[(long)c * taps + j], v, h);
-    }
-    out[(long)t * W + c] = (TO)h;
+  float h = xc;
+  for (int j = 0; j < taps; ++j) {
+    const int d = n - j;             // the input d steps back
+    float v = 0.f;
+    if (d == 0) v = xc;
+    else if (t - d >= a) v = x[(long)(t - d) * W + c];
+    else if (p - d >= 0 && slot >= 0) v = state[((long)slot * n + (n - (d - (t - a)))) * W + c];
+    h = fmaf(w[(long)c * taps + j], v, h);
   }
+  out[(long)t * W + c] = (TO)h;
 }
 
 // one thread per (sequence, channel): entry i of the new history is old entry i + len while that
@@ -109,7 +110,7 @@ __device__ __forceinline__ void row_stats(const float* __restrict__ sy, int W, f
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void post_norm_add_kernel(const float* __restrict__ x, const T* __restrict__ y,
+__global__ __launch_bounds__(1024) void post_norm_add_kernel(const float* __restrict__ x, const T* __restrict__ y,
                                                             const float* __restrict__ nw, const float* __restrict__ nb,
                                                             float eps, const float* __restrict__ scale,
                                                             float* __restrict__ out, T* __restrict__ cast, int W) {
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(256) void post_norm_add_kernel(const float* __restr
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void post_norm_add_avg_kernel(float* __restrict__ x, const T* __restrict__ y,
+__global__ __launch_bounds__(1024) void post_norm_add_avg_kernel(float* __restrict__ x, const T* __restrict__ y,
                                                                 const float* __restrict__ nw,
                                                                 const float* __restrict__ nb, float eps,
                                                                 const float* __restrict__ scale,
@@ -230,7 +231,7 @@ __global__ __launch_bounds__(256) void rope_heads_copy_kernel(const T* __restric
 }
 
 template <typename TO>
-__global__ __launch_bounds__(256) void layer_norm_rows_kernel(const float* __restrict__ x, const float* __restrict__ nw,
+__global__ __launch_bounds__(1024) void layer_norm_rows_kernel(const float* __restrict__ x, const float* __restrict__ nw,
                                                               const float* __restrict__ nb, float eps,
                                                               const long* __restrict__ idx, TO* __restrict__ out,
                                                               int W) {
@@ -246,6 +247,9 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(const float* __res
 
 }  // namespace
 
+// threads of a one-row workgroup: about four elements per thread, whole waves, at most 1024
+static int row_threads(int W) { return std::min(1024, std::max(64, (W / 4 + 63) / 64 * 64)); }
+
 void launch_embed_scaled(const int* ids, const void* table, float scale, float* out, int T, int W, int vocab, bool f32,
                          hipStream_t s) {
   if (T <= 0) return;
@@ -256,10 +260,11 @@ void launch_embed_scaled(const int* ids, const void* table, float scale, float* 
 void launch_conv_mix(const float* x, const float* w, const float* state, const int* state_slots, const int* row_cu,
                      int nseq, const int* positions, void* out, int T, int W, int taps, bool f32, hipStream_t s) {
   if (T <= 0) return;
+  dim3 grid(T, (W + 255) / 256);
   if (f32)
-    conv_mix_kernel<float><<<T, 256, 0, s>>>(x, w, state, state_slots, row_cu, nseq, positions, (float*)out, W, taps);
+    conv_mix_kernel<float><<<grid, 256, 0, s>>>(x, w, state, state_slots, row_cu, nseq, positions, (float*)out, W, taps);
   else
-    conv_mix_kernel<bf16><<<T, 256, 0, s>>>(x, w, state, state_slots, row_cu, nseq, positions, (bf16*)out, W, taps);
+    conv_mix_kernel<bf16><<<grid, 256, 0, s>>>(x, w, state, state_slots, row_cu, nseq, positions, (bf16*)out, W, taps);
 }
 
 void launch_conv_state_update(const float* x, float* state, const int* state_slots, const int* row_cu, int nseq,
@@ -274,9 +279,9 @@ void launch_post_norm_add(const float* x, const void* y, const float* nw, const 
   if (T <= 0) return;
   const size_t sm = (size_t)W * sizeof(float);
   if (f32)
-    post_norm_add_kernel<float><<<T, 256, sm, s>>>(x, (const float*)y, nw, nb, eps, scale, out, (float*)cast, W);
+    post_norm_add_kernel<float><<<T, row_threads(W), sm, s>>>(x, (const float*)y, nw, nb, eps, scale, out, (float*)cast, W);
   else
-    post_norm_add_kernel<bf16><<<T, 256, sm, s>>>(x, (const bf16*)y, nw, nb, eps, scale, out, (bf16*)cast, W);
+    post_norm_add_kernel<bf16><<<T, row_threads(W), sm, s>>>(x, (const bf16*)y, nw, nb, eps, scale, out, (bf16*)cast, W);
 }
 
 void launch_post_norm_add_avg(float* x, const void* y, const float* nw, const float* nb, float eps, const float* scale,
@@ -285,9 +290,9 @@ void launch_post_norm_add_avg(float* x, const void* y, const float* nw, const fl
   if (T <= 0) return;
   const size_t sm = (size_t)W * sizeof(float);
   if (f32)
-    post_norm_add_avg_kernel<float><<<T, 256, sm, s>>>(x, (const float*)y, nw, nb, eps, scale, stack, plane, index, avg, W);
+    post_norm_add_avg_kernel<float><<<T, row_threads(W), sm, s>>>(x, (const float*)y, nw, nb, eps, scale, stack, plane, index, avg, W);
   else
-    post_norm_add_avg_kernel<bf16><<<T, 256, sm, s>>>(x, (const bf16*)y, nw, nb, eps, scale, stack, plane, index, avg, W);
+    post_norm_add_avg_kernel<bf16><<<T, row_threads(W), sm, s>>>(x, (const bf16*)y, nw, nb, eps, scale, stack, plane, index, avg, W);
 }
 
 void launch_latent_prep(const void* z, long z_ld, int Q, int R, int rd, int H, const float* qn_w, const float* kvn_w,
@@ -321,8 +326,8 @@ void launch_layer_norm_rows(const float* x, const float* nw, const float* nb, fl
                             int R, int W, bool f32, hipStream_t s) {
   if (R <= 0) return;
   const size_t sm = (size_t)W * sizeof(float);
-  if (f32) layer_norm_rows_kernel<float><<<R, 256, sm, s>>>(x, nw, nb, eps, idx, (float*)out, W);
-  else layer_norm_rows_kernel<bf16><<<R, 256, sm, s>>>(x, nw, nb, eps, idx, (bf16*)out, W);
+  if (f32) layer_norm_rows_kernel<float><<<R, row_threads(W), sm, s>>>(x, nw, nb, eps, idx, (float*)out, W);
+  else layer_norm_rows_kernel<bf16><<<R, row_threads(W), sm, s>>>(x, nw, nb, eps, idx, (bf16*)out, W);
 }
 
 }  // namespace bfly

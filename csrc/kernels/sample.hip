@@ -425,11 +425,11 @@ void launch_sample_merge(const float* allp, int tp, int rows, int* out, hipStrea
 // Greedy choice over f32 logits (the f32 serving mode): one workgroup per row, the largest
 // logit wins, the lowest index on ties; a row with a non-finite logit gets id -1, score +inf
 // when `check_finite`.
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 sample_greedy_f32_kernel(const float* __restrict__ logits, long row_stride, int V, int vstart,
                          int* __restrict__ out_ids, float* __restrict__ out_scores, int check_finite) {
-  __shared__ float bv[256];
-  __shared__ int bi[256];
+  __shared__ float bv[1024];
+  __shared__ int bi[1024];
   __shared__ int bad;
   const int row = blockIdx.x;
   const float* lr = logits + (long)row * row_stride;
@@ -437,7 +437,7 @@ sample_greedy_f32_kernel(const float* __restrict__ logits, long row_stride, int 
   __syncthreads();
   float v = -INFINITY;
   int id = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += 256) {
+  for (int i = threadIdx.x; i < V; i += 1024) {
     const float x = lr[i];
     if (!(fabsf(x) <= 3.4028235e38f)) bad = 1;
     if (x > v) { v = x; id = i; }
@@ -445,7 +445,7 @@ sample_greedy_f32_kernel(const float* __restrict__ logits, long row_stride, int 
   bv[threadIdx.x] = v;
   bi[threadIdx.x] = id;
   __syncthreads();
-  for (int o = 128; o > 0; o >>= 1) {
+  for (int o = 512; o > 0; o >>= 1) {
     if ((int)threadIdx.x < o) {
       const float ov = bv[threadIdx.x + o];
       const int oi = bi[threadIdx.x + o];
@@ -466,7 +466,7 @@ sample_greedy_f32_kernel(const float* __restrict__ logits, long row_stride, int 
 void launch_sample_greedy_f32(const float* logits, long row_stride, int rows, int V, int vstart, int* out_ids,
                               float* out_scores, hipStream_t stream, int check_finite) {
   if (rows <= 0) return;
-  sample_greedy_f32_kernel<<<rows, 256, 0, stream>>>(logits, row_stride, V, vstart, out_ids, out_scores, check_finite);
+  sample_greedy_f32_kernel<<<rows, 1024, 0, stream>>>(logits, row_stride, V, vstart, out_ids, out_scores, check_finite);
 }
 
 void launch_sample(const bf16* logits, long row_stride, int rows, int V, int vstart,
