@@ -42,36 +42,121 @@ __device__ __forceinline__ int seq_of_row(const int* __restrict__ row_cu, int ns
   return (nseq > 0 && row_cu[lo] <= t && t < row_cu[lo + 1]) ? lo : -1;
 }
 
-// one thread per (row, channel): the taps' loads are independent of one another
-template <typename TO>
+// one thread per (row, V consecutive channels): the taps' loads are independent of one another
+// (V = 4 when the width allows 16-byte accesses)
+template <typename TO, int V>
 __global__ __launch_bounds__(256) void conv_mix_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                        const float* __restrict__ state,
                                                        const int* __restrict__ state_slots,
                                                        const int* __restrict__ row_cu, int nseq,
                                                        const int* __restrict__ positions, TO* __restrict__ out,
                                                        int W, int taps) {
+  typedef float fv __attribute__((ext_vector_type(V)));
   const int t = blockIdx.x;
-  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * V;
   if (c >= W) return;
-  const float xc = x[(long)t * W + c];
+  const fv xc = *reinterpret_cast<const fv*>(x + (long)t * W + c);
   const int s = (w && taps > 0) ? seq_of_row(row_cu, nseq, t) : -1;
-  if (s < 0) {                       // no convolution, or a row outside every sequence
-    out[(long)t * W + c] = (TO)xc;
-    return;
+  fv h = xc;
+  if (s >= 0) {                      // (else: no convolution, or a row outside every sequence)
+    const int a = row_cu[s], p = positions[t];
+    const int slot = state_slots ? state_slots[s] : -1;
+    const int n = taps - 1;
+    for (int j = 0; j < taps; ++j) {
+      const int d = n - j;           // the input d steps back
+      fv v;
+#pragma unroll
+      for (int e = 0; e < V; ++e) v[e] = 0.f;
+      if (d == 0) v = xc;
+      else if (t - d >= a) v = *reinterpret_cast<const fv*>(x + (long)(t - d) * W + c);
+      else if (p - d >= 0 && slot >= 0)
+        v = *reinterpret_cast<const fv*>(state + ((long)slot * n + (n - (d - (t - a)))) * W + c);
+#pragma unroll
+      for (int e = 0; e < V; ++e) h[e] = fmaf(w[(long)(c + e) * taps + j], v[e], h[e]);
+    }
   }
-  const int a = row_cu[s], p = positions[t];
-  const int slot = state_slots ? state_slots[s] : -1;
+#pragma unroll
+  for (int e = 0; e < V; ++e) out[(long)t * W + c + e] = (TO)h[e];
+}
+
+// The same for up to 8 taps with RB consecutive rows per workgroup: a thread keeps the last
+// taps - 1 inputs of its channels in registers and slides over the rows, so a row costs one load
+// of x; the history is fetched anew (earlier rows, the pool, or zeros) at the block's first row
+// and wherever a new sequence begins. Taps are summed in the same order as above.
+template <typename TO, int V>
+__global__ __launch_bounds__(256) void conv_mix_rows_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                            const float* __restrict__ state,
+                                                            const int* __restrict__ state_slots,
+                                                            const int* __restrict__ row_cu, int nseq,
+                                                            const int* __restrict__ positions, TO* __restrict__ out,
+                                                            int W, int taps, int T, int RB) {
+  typedef float fv __attribute__((ext_vector_type(V)));
+  constexpr int MAXN = 7;
+  const int t0 = blockIdx.x * RB, t1 = min(T, t0 + RB);
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * V;
+  if (c >= W) return;
   const int n = taps - 1;
-  float h = xc;
-  for (int j = 0; j < taps; ++j) {
-    const int d = n - j;             // the input d steps back
-    float v = 0.f;
-    if (d == 0) v = xc;
-    else if (t - d >= a) v = x[(long)(t - d) * W + c];
-    else if (p - d >= 0 && slot >= 0) v = state[((long)slot * n + (n - (d - (t - a)))) * W + c];
-    h = fmaf(w[(long)c * taps + j], v, h);
+  fv wv[MAXN + 1], hist[MAXN];
+#pragma unroll
+  for (int j = 0; j <= MAXN; ++j)
+#pragma unroll
+    for (int e = 0; e < V; ++e) wv[j][e] = j < taps ? w[(long)(c + e) * taps + j] : 0.f;
+  int s = -1, send = t0;
+  bool fetch = true;
+  for (int t = t0; t < t1; ++t) {
+    if (t >= send) {
+      s = seq_of_row(row_cu, nseq, t);
+      send = s >= 0 ? row_cu[s + 1] : t + 1;
+      fetch = true;
+    }
+    const fv xc = *reinterpret_cast<const fv*>(x + (long)t * W + c);
+    fv h = xc;
+    if (s >= 0) {
+      if (fetch) {
+        const int a = row_cu[s], p = positions[t];
+        const int slot = state_slots ? state_slots[s] : -1;
+#pragma unroll
+        for (int k = 0; k < MAXN; ++k) {
+          if (k >= n) break;
+          const int d = n - k;
+          fv v;
+#pragma unroll
+          for (int e = 0; e < V; ++e) v[e] = 0.f;
+          if (t - d >= a) v = *reinterpret_cast<const fv*>(x + (long)(t - d) * W + c);
+          else if (p - d >= 0 && slot >= 0)
+            v = *reinterpret_cast<const fv*>(state + ((long)slot * n + (n - (d - (t - a)))) * W + c);
+          hist[k] = v;
+        }
+        fetch = false;
+      }
+#pragma unroll
+      for (int k = 0; k < MAXN; ++k) {
+        if (k >= n) break;
+#pragma unroll
+        for (int e = 0; e < V; ++e) h[e] = fmaf(wv[k][e], hist[k][e], h[e]);
+      }
+#pragma unroll
+      for (int k = 0; k <= MAXN; ++k)
+        if (k == n) {
+#pragma unroll
+          for (int e = 0; e < V; ++e) h[e] = fmaf(wv[k][e], xc[e], h[e]);
+        }
+#pragma unroll
+      for (int k = 0; k < MAXN; ++k) {
+        if (k + 1 < n) hist[k] = hist[k + 1];
+        else if (k + 1 == n) hist[k] = xc;
+      }
+    }
+    if constexpr (V == 4 && sizeof(TO) == 2) {
+      bf16x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (bf16)h[e];
+      *reinterpret_cast<bf16x4*>(out + (long)t * W + c) = o;
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) out[(long)t * W + c + e] = (TO)h[e];
+    }
   }
-  out[(long)t * W + c] = (TO)h;
 }
 
 // one thread per (sequence, channel): entry i of the new history is old entry i + len while that
@@ -260,11 +345,22 @@ void launch_embed_scaled(const int* ids, const void* table, float scale, float* 
 void launch_conv_mix(const float* x, const float* w, const float* state, const int* state_slots, const int* row_cu,
                      int nseq, const int* positions, void* out, int T, int W, int taps, bool f32, hipStream_t s) {
   if (T <= 0) return;
+  if (w && taps >= 1 && taps <= 8) {
+    // rows per workgroup: one for steps of few rows (every row its own sequence, as in decoding)
+    const int RB = std::min(16, std::max(1, T / 512));
+#define BFLY_CONV(TO, V)                                                                                     \
+  conv_mix_rows_kernel<TO, V><<<dim3((T + RB - 1) / RB, (W / V + 255) / 256), 256, 0, s>>>(                  \
+      x, w, state, state_slots, row_cu, nseq, positions, (TO*)out, W, taps, T, RB)
+    if (W % 4 == 0) { if (f32) BFLY_CONV(float, 4); else BFLY_CONV(bf16, 4); }
+    else { if (f32) BFLY_CONV(float, 1); else BFLY_CONV(bf16, 1); }
+#undef BFLY_CONV
+    return;
+  }
   dim3 grid(T, (W + 255) / 256);
   if (f32)
-    conv_mix_kernel<float><<<grid, 256, 0, s>>>(x, w, state, state_slots, row_cu, nseq, positions, (float*)out, W, taps);
+    conv_mix_kernel<float, 1><<<grid, 256, 0, s>>>(x, w, state, state_slots, row_cu, nseq, positions, (float*)out, W, taps);
   else
-    conv_mix_kernel<bf16><<<grid, 256, 0, s>>>(x, w, state, state_slots, row_cu, nseq, positions, (bf16*)out, W, taps);
+    conv_mix_kernel<bf16, 1><<<grid, 256, 0, s>>>(x, w, state, state_slots, row_cu, nseq, positions, (bf16*)out, W, taps);
 }
 
 void launch_conv_state_update(const float* x, float* state, const int* state_slots, const int* row_cu, int nseq,

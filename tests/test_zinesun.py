@@ -87,7 +87,7 @@ def test_scaled_embedding(target):
     assert got.dtype == torch.float32 and close(got, O.scaled_embedding(table, ids, 3.25), torch.float32)
 
 
-@pytest.mark.parametrize("taps", [1, 2, 3, 5])
+@pytest.mark.parametrize("taps", [1, 2, 3, 5, 9])
 def test_input_convolution_over_steps_and_slots(target, taps):
     """Three sequences fed in portions (one token, two tokens, longer than the kernel, shorter
     than it), interleaved in packed steps, through two history slots of which one is handed from a
@@ -122,6 +122,36 @@ def test_input_convolution_over_steps_and_slots(target, taps):
             at[n] += c
             r += c
     assert all(at[n] == len(seqs[n]) for n in seqs)
+
+
+@pytest.mark.parametrize("taps,C", [(4, 64), (3, 50), (8, 24)])
+def test_input_convolution_long_steps(target, taps, C):
+    """Steps of more than a thousand rows (several rows per workgroup slide over sequence starts,
+    one-row sequences and an empty one), continued from a first step's history."""
+    dev, dt = target
+    g = torch.Generator().manual_seed(taps + C)
+    w = bf(0.5 * torch.randn(C, taps, generator=g, dtype=F64))
+    lens = {"a": 1500, "b": 3, "c": 1, "d": 900}
+    seqs = {n: torch.randn(L, C, generator=g, dtype=F64).float().to(F64) for n, L in lens.items()}
+    want = {n: O.causal_conv_residual(x, w) for n, x in seqs.items()}
+    state = torch.full((4, taps - 1, C), -3.0, dtype=torch.float32, device=dev)
+    slot = {"a": 2, "b": 0, "c": 3, "d": 1}
+    at = {n: 0 for n in seqs}
+    for step in ([("a", 2), ("d", 1)], [("b", 3), ("a", 1098), ("c", 1), ("d", 0), ("d", 899)], [("a", 400)]):
+        rows, cu, pos, sl = [], [0], [], []
+        for n, c in step:
+            rows.append(seqs[n][at[n]:at[n] + c])
+            pos += list(range(at[n], at[n] + c))
+            cu.append(cu[-1] + c)
+            sl.append(slot[n])
+        x = torch.cat(rows).to(dev, torch.float32)
+        h = ops.conv_mix(x, w.to(dev, torch.float32), state, i32(sl, dev), i32(cu, dev), i32(pos, dev), dt)
+        ops.conv_state_update_(x, state, i32(sl, dev), i32(cu, dev), i32(pos, dev))
+        r = 0
+        for n, c in step:
+            assert c == 0 or close(h[r:r + c], want[n][at[n]:at[n] + c], dt, bf16_tol=1e-2), (n, at[n], c)
+            at[n] += c
+            r += c
 
 
 def test_convolution_leaves_padding_sequences_alone(target):
