@@ -99,7 +99,8 @@ def build_parser() -> argparse.ArgumentParser:
                     help="instead of the headline run: prefill and decode throughput of a Nesizen stack "
                          "(windowed attention, shared keys, gated linear attention, sigmoid MoE) beside a "
                          "Mixtral stack of equal width, depth, heads and experts, random weights, one GPU; "
-                         "SIZES = comma list of s, m, l (width 1024 / 2048 / 4096)")
+                         "SIZES = comma list of s, m, l (width 1024 / 2048 / 4096); --mixer-family chooses the "
+                         "family that is timed")
     return ap
 
 
