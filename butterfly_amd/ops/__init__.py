@@ -732,10 +732,23 @@ def moe_gate_scale_(h, gates, e0: int, num_local: int):
 ACTS = {"none": 0, "relu2": 1, "xielu": 2}
 
 
-def _mfma_gemm_ok(x, w, out_dtype) -> bool:
-    """The MFMA GEMM family takes bf16 operands with K % 64 == 0, N % 128 == 0 and 16-byte rows."""
-    return (x.dtype == torch.bfloat16 and out_dtype in (None, torch.bfloat16) and w.shape[1] % 64 == 0
-            and w.shape[0] % 128 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and x.shape[0] > 0)
+_tuned_ok: dict = {}
+
+
+def _mfma_gemm_ok(x, w, out_dtype, bias=None) -> bool:
+    """The tuned MFMA GEMM family takes bf16 operands with K % 64 == 0, N % 128 == 0 and 16-byte
+    rows, when the plan it would choose for (M, N, K) accepts the shape (a dry run, cached: a
+    shallow K can be too short for the plan's split or pipeline depth)."""
+    if not (x.dtype == torch.bfloat16 and out_dtype in (None, torch.bfloat16) and w.shape[1] % 64 == 0
+            and w.shape[0] % 128 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and x.shape[0] > 0
+            and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0):
+        return False
+    key = (x.shape[0], w.shape[0], w.shape[1], bias is not None)
+    ok = _tuned_ok.get(key)
+    if ok is None:
+        ok = _tuned_ok[key] = torch.ops.bfly.gemm_check(key[0], key[1], key[2],
+                                                       EPILOGUES["bias" if bias is not None else "none"]) == 0
+    return ok
 
 
 def linear_act(x, w, bias=None, act: str = "none", out_dtype=None, act_params=None):
@@ -747,7 +760,7 @@ def linear_act(x, w, bias=None, act: str = "none", out_dtype=None, act_params=No
     if not _gpu(x):
         return ref.linear_act(x, w, bias, act, out_dtype, act_params)
     a0, a1 = (float(act_params[0]), float(act_params[1])) if act == "xielu" else (0.0, 0.0)
-    if _mfma_gemm_ok(x, w, out_dtype):
+    if _mfma_gemm_ok(x, w, out_dtype, bias):
         y = linear(x, w, bias=bias)
         if act != "none":
             torch.ops.bfly.act_(y, ACTS[act], a0, a1)

@@ -201,7 +201,7 @@ def test_post_norm_residual_and_depth_average(target, T, C):
     assert close(stack[5], x2, torch.float32) and close(xx, O.depth_average(prev + [want, x2], avg2), torch.float32)
 
 
-@pytest.mark.parametrize("M,N,K", [(5, 7, 13), (70, 130, 50), (3, 256, 128), (600, 384, 192)])
+@pytest.mark.parametrize("M,N,K", [(5, 7, 13), (70, 130, 50), (3, 256, 128), (600, 384, 192), (260, 256, 64), (16, 128, 64)])
 def test_xielu_projection(target, M, N, K):
     dev, dt = target
     g = torch.Generator().manual_seed(M + N)
