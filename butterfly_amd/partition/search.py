@@ -46,6 +46,10 @@ def factorizations(n: int) -> list[tuple[int, int, int]]:
 
 
 def _tp_ok(cfg: ModelConfig, tp: int) -> bool:
+    if tp == 1:
+        return True
+    if cfg.layer_specs:          # heterogeneous stacks run unsharded (data-parallel replicas only)
+        return False
     if cfg.num_heads % tp:
         return False
     if not (cfg.num_kv_heads % tp == 0 or tp % cfg.num_kv_heads == 0):
@@ -141,12 +145,12 @@ def partition(cfg: Union[ModelConfig, str], n_gpus: int, strategy: Union[str, di
     for dp, tp, pp in factorizations(n_gpus):
         if any(fixed.get(k, v) != v for k, v in (("dp", dp), ("tp", tp), ("pp", pp))):
             continue
-        if not _tp_ok(cfg, tp) or pp > cfg.num_layers:
+        if not _tp_ok(cfg, tp) or pp > cfg.num_layers or (cfg.layer_specs and pp > 1):
             continue
         eps = [1]
         # expert parallelism spans the DP replicas (per pipeline stage when pp > 1: the
         # asynchronous pipeline keeps each stage's EP group in lockstep)
-        if cfg.is_moe and dp > 1 and cfg.num_experts % dp == 0 and tp == 1:
+        if cfg.is_moe and dp > 1 and cfg.num_experts % dp == 0 and tp == 1 and not cfg.layer_specs:
             eps.append(dp)
         if "ep" in fixed:
             eps = [e for e in eps if e == fixed["ep"]]

@@ -560,3 +560,23 @@ def test_random_init_and_registry():
                                                 dtype="fp32", async_decode=False), model=m, device=torch.device("cpu"))
     out = eng.generate([[1, 2, 3], [4]], SamplingParams(max_tokens=3, temperature=0.0, ignore_eos=True))
     assert [len(o) for o in out] == [3, 3]
+
+
+def test_llm_entry_point_from_a_model_folder(tmp_path):
+    """butterfly_amd.LLM on a folder: family chosen by config.json, a data-parallel-only plan from
+    the partitioner, the default (overlapped) engine settings, greedy tokens equal the oracle's."""
+    from butterfly_amd.api import LLM
+
+    cfg = cfg_b()
+    W = O.random_weights(cfg, seed=21)
+    d = tmp_path / "model"
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in W.items()}, str(d / "model.safetensors"))
+    llm = LLM(str(d), engine_config=EngineConfig(max_batch=3, max_seq_len=96, kv_cache_tokens=256, dtype="fp32"))
+    assert llm.cfg.arch == "zinesun" and (llm.plan.mesh.tp, llm.plan.mesh.pp) == (1, 1)
+    prompts = [tokens_of(cfg, n, 60 + n) for n in (9, 33, 2)]
+    outs = llm.generate(prompts, SamplingParams(max_tokens=5, temperature=0.0, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        assert o.token_ids == O.greedy(cfg, W, p, 5)
+    llm.close()
