@@ -313,6 +313,47 @@ def test_shared_head_attention_edges(target, H, D, Dv, window):
     assert close(got2, want, dt, f32_tol=1e-4, bf16_tol=4e-2)
 
 
+@pytest.mark.parametrize("H,D,Dv,window", [(16, 96, 64, 2000), (5, 256, 192, 700), (8, 40, 24, 640)])
+def test_shared_head_attention_decoding_long_contexts(target, H, D, Dv, window):
+    """Decoded rows only, over hundreds of cached tokens: the shape whose pages the matrix-core
+    form splits over several workgroups and merges. One key far back and the key at the window's
+    edge stand out for some heads."""
+    dev, dt = target
+    bs = 32
+    g = torch.Generator().manual_seed(H + window)
+    rnd = lambda *s: bf(torch.randn(*s, generator=g, dtype=F64))        # noqa: E731
+    lens = [1000, 641, 33, 900]
+    seqs = [(0.3 * rnd(L, D), rnd(L, Dv)) for L in lens]
+    q = 0.3 * rnd(len(lens), H, D)
+    for s, L in enumerate(lens):
+        i = L - 1
+        for h, j in ((0, max(0, i - window + 1)), (1, i - window), (2, 5), (3, i)):
+            if h < H and 0 <= j <= i:
+                u = rnd(D)
+                u = u / u.norm()
+                seqs[s][0][j] = bf(4.0 * u)
+                q[s, h] = bf(6.0 * u)
+    pos = [L - 1 for L in lens]
+    cu = list(range(len(lens) + 1))
+    gate = torch.rand(len(lens), H, generator=g, dtype=F64).float().to(F64)
+    kc, vc, tables = paged(seqs, ops.attn_window_pad(D, dt), ops.attn_window_pad(Dv, dt), bs, dev, dt,
+                           lambda n: torch.randperm(n, generator=g).tolist())
+    qd = torch.zeros(len(lens), H, kc.shape[3], dtype=dt, device=dev)
+    qd[:, :, :D] = q.to(dev, dt)
+    want = torch.zeros(len(lens), H, Dv, dtype=F64)
+    for s, L in enumerate(lens):
+        k, v = seqs[s]
+        for h in range(H):
+            full = torch.zeros(L, D, dtype=F64)
+            full[L - 1] = q[s, h]
+            want[s, h] = O.windowed_softmax_attention(full, k, v, 0.7, window)[L - 1]
+    want = want * gate[:, :, None]
+    for fold in (True, False):
+        got = ops.attn_window_paged(qd, kc, vc, tables, i32(cu, dev), i32(pos, dev), 0.7, window, 0, None,
+                                    fold_heads=fold, out_scale=gate.to(dev, torch.float32))[:, :, :Dv]
+        assert close(got, want, dt, f32_tol=1e-4, bf16_tol=4e-2), fold
+
+
 def test_latent_preparation_and_cache_append(target):
     dev, dt = target
     g = torch.Generator().manual_seed(9)
