@@ -335,6 +335,159 @@ __global__ __launch_bounds__(256) void attn_window_mfma_kernel(const bf16* __res
   }
 }
 
+// Folded form for steps of many rows (prompts), one shared key / value head: a workgroup owns 64
+// consecutive (token, head) rows of a sequence, 16 per wave, and walks the union of their visible
+// pages once. Each page's K rows and transposed V rows are staged in LDS by all four waves
+// (double buffered: the next page travels to registers while the current one is multiplied, one
+// barrier per page), so a page is read from memory once per 64 rows instead of once per 16, and
+// every wave keeps its own rows' online softmax: no merge at the end. Rows pitch D + 8 (K) and
+// 32 + 4 (V^T) elements keep the 16-byte / 8-byte fragment reads off a common bank.
+template <int DS, int DVT>
+__global__ __launch_bounds__(256) void attn_fold_tile_kernel(const bf16* __restrict__ q, long q_ld,
+                                                             const bf16* __restrict__ k_cache,
+                                                             const bf16* __restrict__ v_cache,
+                                                             const int* __restrict__ tables, int max_blocks,
+                                                             const int* __restrict__ row_cu, int nseq,
+                                                             const int* __restrict__ positions, float scale,
+                                                             int window, int keep_first,
+                                                             const float* __restrict__ sink,
+                                                             const float* __restrict__ out_scale,
+                                                             bf16* __restrict__ out, int H) {
+  constexpr int D = 32 * DS, Dv = 16 * DVT, BS = 32, KP = D + 8, VP = BS + 4;
+  constexpr int NK = BS * D / 8, NV = Dv * BS / 8;            // 16-byte segments of a page
+  constexpr int NKS = (NK + 255) / 256, NVS = (NV + 255) / 256;
+  extern __shared__ __attribute__((aligned(16))) unsigned char fold_smem[];
+  bf16* Ks = reinterpret_cast<bf16*>(fold_smem);            // [2][BS][KP]
+  bf16* Vs = Ks + 2 * BS * KP;                                // [2][Dv][VP]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int tile = blockIdx.x;
+  int s = 0, row0 = 0, rend = 0;
+  for (; s < nseq; ++s) {
+    const int a = row_cu[s] * H, b = row_cu[s + 1] * H;
+    const int nt = (b - a + 63) >> 6;
+    if (tile < nt) { row0 = a + 64 * tile; rend = b; break; }
+    tile -= nt;
+  }
+  if (s >= nseq) return;                   // (the whole workgroup)
+  const int qr = lane & 15, gg = lane >> 4;
+  const bool rv = row0 + 16 * wave + qr < rend;
+  const long frow = rv ? row0 + 16 * wave + qr : row0;
+  const long row = frow / H;
+  const int h = (int)(frow % H);
+  const int p = rv ? positions[row] : -1;
+  // positions grow along a sequence's rows: the tile's first and last rows bound them
+  const int pmin = positions[row0 / H], pmax = positions[(min(rend, row0 + 64) - 1) / H];
+  bf16x8 qf[DS];
+#pragma unroll
+  for (int ds = 0; ds < DS; ++ds)
+    qf[ds] = *reinterpret_cast<const bf16x8*>(q + row * q_ld + (long)h * D + 32 * ds + 8 * gg);
+  const int* tab = tables + (long)s * max_blocks;
+  float m = sink ? sink[h] : -1e30f, l = sink ? 1.f : 0.f;
+  f32x4 o[DVT];
+#pragma unroll
+  for (int t = 0; t < DVT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int kp = (min(keep_first, pmax + 1) + BS - 1) / BS;          // pages of the kept prefix
+  const int wp0 = max(max(0, pmin - window + 1) / BS, kp), wp1 = pmax / BS;
+  const int npages = kp + max(0, wp1 - wp0 + 1);
+  auto page_of = [&](int i) { return i < kp ? i : wp0 + (i - kp); };
+  bf16x8 kreg[NKS], vreg[NVS];
+  auto gload = [&](int pg) {
+    const long blk = tab[pg];
+    const bf16* Kp = k_cache + blk * BS * D;
+    const bf16* Vp = v_cache + blk * Dv * BS;
+#pragma unroll
+    for (int i = 0; i < NKS; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < NK) kreg[i] = *reinterpret_cast<const bf16x8*>(Kp + (long)idx * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < NVS; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < NV) vreg[i] = *reinterpret_cast<const bf16x8*>(Vp + (long)idx * 8);
+    }
+  };
+  auto sstore = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < NKS; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < NK) *reinterpret_cast<bf16x8*>(Ks + (long)(buf * BS + idx / (D / 8)) * KP + 8 * (idx % (D / 8))) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NVS; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < NV) {
+        bf16* dst = Vs + (long)(buf * Dv + idx / 4) * VP + 8 * (idx & 3);       // 8-byte aligned rows
+        const bf16x8 v = vreg[i];
+        *reinterpret_cast<bf16x4*>(dst) = bf16x4{v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<bf16x4*>(dst + 4) = bf16x4{v[4], v[5], v[6], v[7]};
+      }
+    }
+  };
+  if (npages > 0) gload(page_of(0));
+  for (int pi = 0; pi < npages; ++pi) {
+    const int buf = pi & 1;
+    sstore(buf);
+    __syncthreads();      // the page is in LDS; every wave has left the buffer written next
+    if (pi + 1 < npages) gload(page_of(pi + 1));
+    const int pg = page_of(pi);
+    const bf16* Kb = Ks + (long)buf * BS * KP;
+    const bf16* Vb = Vs + (long)buf * Dv * VP;
+    f32x4 st[2];
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) {
+      st[kh] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ds = 0; ds < DS; ++ds)
+        st[kh] = mfma16(*reinterpret_cast<const bf16x8*>(Kb + (16 * kh + qr) * KP + 32 * ds + 8 * gg), qf[ds], st[kh]);
+    }
+    float sc[8], mx = -INFINITY;
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int j = pg * BS + 16 * kh + 4 * gg + i;
+        const bool ok = j <= p && (p - j < window || j < keep_first);
+        sc[4 * kh + i] = ok ? st[kh][i] * scale : -INFINITY;
+        mx = fmaxf(mx, sc[4 * kh + i]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mn = fmaxf(m, mx);
+    const float corr = __expf(m - mn);
+    float rs = 0.f;
+    bf16x8 pb;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float pe = __expf(sc[e] - mn);      // exp(-inf) = 0 for masked keys
+      rs += pe;
+      pb[e] = (bf16)pe;
+    }
+    rs += __shfl_xor(rs, 16, 64);
+    rs += __shfl_xor(rs, 32, 64);
+    l = l * corr + rs;
+    m = mn;
+#pragma unroll
+    for (int t = 0; t < DVT; ++t) {
+      const bf16* vr = Vb + (16 * t + qr) * VP + 4 * gg;
+      const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vr);
+      const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vr + 16);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[t][i] *= corr;
+      o[t] = mfma16(bf16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]}, pb, o[t]);
+    }
+  }
+  if (!rv) return;
+  const float inv = (out_scale ? out_scale[row * H + h] : 1.f) / l;
+  bf16* orow = out + (row * H + h) * Dv;
+#pragma unroll
+  for (int t = 0; t < DVT; ++t) {
+    bf16x4 w;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (bf16)(o[t][i] * inv);
+    *reinterpret_cast<bf16x4*>(orow + 16 * t + 4 * gg) = w;
+  }
+}
+
 // One wave per (row, head): fold the nsplit partial results part[split][row][o (Dv) | m | l].
 __global__ __launch_bounds__(64) void attn_split_merge_kernel(const float* __restrict__ part, long part_rows,
                                                               int nsplit, const float* __restrict__ out_scale,
@@ -518,6 +671,33 @@ static bool attn_mfma_dv(const bf16* q, long q_ld, const bf16* kc, const bf16* v
                          const int* row_cu, int nseq, const int* positions, float scale, int window, int keep_first,
                          const float* sink, const float* out_scale, bf16* out, int T, int H, int G, int Dv, bool fold,
                          int nsplit, float* part, hipStream_t s) {
+  if (fold && (long)T * H >= 2048 && (long)T * H >= 128L * nseq) {
+    // many rows per sequence (prompts): 64-row tiles over pages staged in LDS
+    const unsigned tiles = (unsigned)(((long)T * H + 63) / 64 + nseq);
+#define BFLY_ATF(DVT)                                                                                         \
+  {                                                                                                           \
+    constexpr size_t lds = 2 * (32 * (32 * DS + 8) + 16 * DVT * 36) * sizeof(bf16);                           \
+    static bool once = false;                                                                                 \
+    if (!once) {                                                                                              \
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fold_tile_kernel<DS, DVT>),               \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                        \
+      once = true;                                                                                            \
+    }                                                                                                         \
+    attn_fold_tile_kernel<DS, DVT><<<tiles, 256, lds, s>>>(q, q_ld, kc, vc, tables, max_blocks, row_cu, nseq,   \
+                                                          positions, scale, window, keep_first, sink, out_scale, \
+                                                          out, H);                                            \
+  }
+    switch (Dv) {
+      case 32: BFLY_ATF(2); return true;
+      case 64: BFLY_ATF(4); return true;
+      case 96: BFLY_ATF(6); return true;
+      case 128: BFLY_ATF(8); return true;
+      case 192: BFLY_ATF(12); return true;
+      case 256: BFLY_ATF(16); return true;
+      default: return false;
+    }
+#undef BFLY_ATF
+  }
   // one workgroup per 16-row tile; every sequence adds at most one partly filled tile
   dim3 grid(((fold ? T * H : T) + 15) / 16 + nseq, fold ? 1 : H, nsplit);
   const int fd = fold ? H : 0;
