@@ -263,7 +263,7 @@ def paged(seq_rows, width_k, width_v, bs, dev, dt, order):
 
 @pytest.mark.parametrize("H,D,Dv,window", [(3, 20, 12, 9), (5, 96, 64, 33), (16, 128, 96, 40), (2, 32, 32, 1),
                                           (4, 64, 64, 500), (16, 96, 64, 33), (32, 64, 32, 9), (16, 256, 192, 100),
-                                          (24, 192, 128, 64)])
+                                          (24, 192, 128, 64), (16, 256, 256, 77)])
 def test_shared_head_attention_edges(target, H, D, Dv, window):
     """Folded multi-query attention over one shared cached head, no sink, with an output gate. A
     long prompt chunk, a short chunk and decoded rows in one packed step. For chosen rows one key
