@@ -24,8 +24,9 @@
 
 Every size and constant comes from the config; the residual, norms, softmax, rotary angles, router
 and gates run in f32 in the bf16 model too. Unsharded (tp = pp = ep = 1). Prompt chunks always
-attend through the paged cache, so one attention kernel serves fresh prompts, continuation chunks
-and decoded tokens.
+attend through the paged cache, so one attention op serves fresh prompts, continuation chunks and
+decoded tokens (its kernel forms share one mask rule: which one runs changes a result only by
+rounding).
 """
 from __future__ import annotations
 
